@@ -2,7 +2,8 @@
 
 A model's cache units (one per entry of the model's run order that writes keys
 and values) are sorted into *groups* by what they need: every key of the request
-(``window=None``) or only the last ``window`` of them. Each group has a pool of
+(``window=None``), only the last ``window`` of them, or (``chunk``) only those of
+the query's own block of ``chunk`` positions. Each group has a pool of
 pages of its own and each request has one block table per group, so a page id
 means the same place in every unit of its group.
 
@@ -50,6 +51,19 @@ class PagedGroupSpec:
     page_size: int                  # tokens in a page
     num_pages: int                  # pages in this group's pool
     window: int | None = None       # None: all keys are kept; n: a query sees the last n keys (itself included)
+    chunk: int | None = None        # n: a query sees the keys of its own block of n positions (counted from 0) only
+
+    @property
+    def keeps_all(self) -> bool:
+        return self.window is None and self.chunk is None
+
+    def first_needed(self, position: int) -> int:
+        """The oldest key that the query at ``position`` sees."""
+        if self.chunk is not None:
+            return position - position % self.chunk
+        if self.window is not None:
+            return position - self.window + 1
+        return 0
 
     def __post_init__(self):
         if self.page_size <= 0:
@@ -58,6 +72,8 @@ class PagedGroupSpec:
             raise ValueError("num_pages must be positive")
         if self.window is not None and self.window <= 0:
             raise ValueError("window must be positive")
+        if self.chunk is not None and (self.chunk <= 0 or self.window is not None):
+            raise ValueError("chunk must be positive and comes without a window")
 
 
 class PageAllocator:
@@ -157,7 +173,7 @@ class CacheManager:
     def __init__(self, groups: list[PagedGroupSpec], num_state_slots: int, share_prefixes: bool = False):
         if not groups:
             raise ValueError("at least one paged group is needed")
-        if share_prefixes and (len(groups) != 1 or groups[0].window is not None):
+        if share_prefixes and (len(groups) != 1 or not groups[0].keeps_all):
             # a page of a windowed group does not stay, and a second group would need the same hits
             raise ValueError("prefixes can be shared only when every layer keeps all keys (one group, no window)")
         self.groups = list(groups)
@@ -305,8 +321,8 @@ class CacheManager:
 
     def commit(self, request_id, new_len: int, new_tokens: Sequence[int] | None = None) -> list[list[int]]:
         """The step that stored the tokens below ``new_len`` has been issued.
-        Pages of a windowed group whose every key lies before the window of the
-        next query (position ``new_len``) are given back. Returns the pages given
+        Pages of a windowed or chunked group whose every key lies before what the
+        next query (position ``new_len``) sees are given back. Returns the pages given
         back, per group. With shared prefixes ``new_tokens`` are the tokens that
         the step stored; pages that they filled become known by their content
         (block_manager.py:811-825)."""
@@ -332,9 +348,9 @@ class CacheManager:
         rc.num_tokens = new_len
         given_back: list[list[int]] = [[] for _ in self.groups]
         for gi, g in enumerate(self.groups):
-            if g.window is None:
+            if g.keeps_all:
                 continue
-            first_needed = new_len - g.window + 1          # oldest key the next query sees
+            first_needed = g.first_needed(new_len)         # oldest key the next query sees
             if first_needed <= 0:
                 continue
             passed = first_needed // g.page_size           # logical pages wholly before it
@@ -351,7 +367,7 @@ class CacheManager:
         its turn and is run again). Pages stay reserved. Not with windows (their pages may be gone) and not with
         shared prefixes (pages may have become known by a content that is taken back)."""
         rc = self.requests[request_id]
-        if self.share_prefixes or any(g.window is not None for g in self.groups):
+        if self.share_prefixes or not all(g.keeps_all for g in self.groups):
             raise CacheError("rewind: not with windows or shared prefixes")
         if not 0 <= new_len <= rc.num_tokens:
             raise CacheError(f"request {request_id!r}: rewind to {new_len} from {rc.num_tokens}")

@@ -39,6 +39,9 @@ class Architecture:
     checkpoint_names: Callable                  # typed configuration -> {checkpoint tensor name: WeightSource}
     ignored_prefixes: tuple[str, ...] = ()      # checkpoint names under these are skipped (nanovllm/utils/loader.py:27-31)
     named_shapes: dict = field(default_factory=dict)   # name -> config.json contents, for measurements and examples
+    # True: ``parse_config(raw, shapes)`` also gets {tensor name: shape} of the checkpoint where there is one (sizes
+    # that config.json does not name and only the stored tensors show)
+    reads_checkpoint_shapes: bool = False
 
 
 _ARCHITECTURES: dict[str, Architecture] = {}
@@ -95,6 +98,8 @@ def resolve_architecture(raw_config: dict) -> Architecture:
     that is registered, else by ``model_type``; a ``model_type`` whose entry is not
     among the listed architectures is an error (registry.py:69-95)."""
     listed = list(raw_config.get("architectures") or [])
+    if isinstance(raw_config.get("architecture"), str):       # a config.json that names its one architecture so
+        listed.append(raw_config["architecture"])
     model_type = raw_config.get("model_type")
     for name in listed:
         arch = _get(name)

@@ -2,7 +2,9 @@
 // and groups, in float or bfloat16 (float scores, running maximum, sum and output).
 // One wave per (token, query head): prompt portions and single decoded tokens are
 // the same case. The query at position p of request r reads the keys at positions
-// lo..p, lo = max(0, p - window + 1) (window 0: lo = 0), of r's block table.
+// lo..p of r's block table: lo = max(0, p - window + 1) with a window, lo = p - p % chunk
+// with a chunk (the keys of p's own block of ``chunk`` positions, counted from the
+// start of the request), else 0. Value heads may have another size (E) than key heads (D).
 // Keys are taken in blocks of 64 aligned to absolute positions, always in rising
 // order, so the result for a position does not depend on the batch or the portion.
 // This is the attention of the 32-bit path and the fallback of the bfloat16 path.
@@ -15,7 +17,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
     const int* __restrict__ token_req, const int* __restrict__ positions, const int* __restrict__ block_tables,
-    int max_blocks, int n_items, int Hq, int Hkv, int D, int page_size, float scale, int window) {
+    int max_blocks, int n_items, int Hq, int Hkv, int D, int E, int page_size, float scale, int window, int chunk) {
   extern __shared__ float q_s[];            // 4 waves x D floats
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + wave;
@@ -31,7 +33,7 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
   const int pos = positions[t];
   const int req = token_req[t];
   const int kvh = h / (Hq / Hkv);
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = chunk > 0 ? pos - pos % chunk : (window > 0 ? max(0, pos - window + 1) : 0);
   const int* bt = block_tables + (size_t)req * max_blocks;
 
   float m = -INFINITY, l = 0.f;
@@ -64,32 +66,33 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
       const float pj = __shfl(p, j, NHV_WAVE);
       const int sj = __shfl(slot, j, NHV_WAVE);
       if (pj == 0.f) continue;                     // same for the whole wave; also skips keys before the window
-      const T* vr = v_cache + ((size_t)sj * Hkv + kvh) * D;
+      const T* vr = v_cache + ((size_t)sj * Hkv + kvh) * E;
 #pragma unroll
       for (int i = 0; i < MAX_D_CHUNKS; ++i) {
         const int d = lane + i * NHV_WAVE;
-        if (d < D) acc[i] = fmaf(pj, to_f32(vr[d]), acc[i]);
+        if (d < E) acc[i] = fmaf(pj, to_f32(vr[d]), acc[i]);
       }
     }
   }
   const float inv = 1.0f / l;
-  T* o = out + ((size_t)t * Hq + h) * D;
+  T* o = out + ((size_t)t * Hq + h) * E;
 #pragma unroll
   for (int i = 0; i < MAX_D_CHUNKS; ++i) {
     const int d = lane + i * NHV_WAVE;
-    if (d < D) o[d] = from_f32<T>(acc[i] * inv);
+    if (d < E) o[d] = from_f32<T>(acc[i] * inv);
   }
 }
 
 extern "C" int nhv_paged_attention_generic(const void* q, const void* k_cache, const void* v_cache, void* out,
                                            const void* token_req, const void* positions, const void* block_tables,
-                                           int max_blocks, int T, int Hq, int Hkv, int D, int page_size, float scale,
-                                           int window, int dtype, void* stream) {
+                                           int max_blocks, int T, int Hq, int Hkv, int D, int E, int page_size,
+                                           float scale, int window, int chunk, int dtype, void* stream) {
   NHV_REQUIRE(T > 0 && Hq > 0 && Hkv > 0 && D > 0 && page_size > 0 && max_blocks > 0,
               "attention: bad sizes T=%d Hq=%d Hkv=%d D=%d page=%d blocks=%d", T, Hq, Hkv, D, page_size, max_blocks);
   NHV_REQUIRE(Hq % Hkv == 0, "attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   NHV_REQUIRE(D <= 64 * MAX_D_CHUNKS, "attention: head size %d is beyond this kernel's limit of %d", D, 64 * MAX_D_CHUNKS);
-  NHV_REQUIRE(window >= 0, "attention: negative window");
+  NHV_REQUIRE(E > 0 && E <= 64 * MAX_D_CHUNKS, "attention: value head size %d is beyond this kernel's limit of %d", E, 64 * MAX_D_CHUNKS);
+  NHV_REQUIRE(window >= 0 && chunk >= 0 && !(window > 0 && chunk > 0), "attention: window %d and chunk %d", window, chunk);
   const long long n_items = (long long)T * Hq;
   NHV_REQUIRE(n_items < (1ll << 31), "attention: too many (token, head) pairs");
   const unsigned blocks = (unsigned)((n_items + 3) / 4);
@@ -98,13 +101,13 @@ extern "C" int nhv_paged_attention_generic(const void* q, const void* k_cache, c
   if (dtype == NHV_F32)
     hipLaunchKernelGGL(paged_attention_generic_kernel<float>, dim3(blocks), dim3(256), lds, s, (const float*)q,
                        (const float*)k_cache, (const float*)v_cache, (float*)out, (const int*)token_req,
-                       (const int*)positions, (const int*)block_tables, max_blocks, (int)n_items, Hq, Hkv, D, page_size,
-                       scale, window);
+                       (const int*)positions, (const int*)block_tables, max_blocks, (int)n_items, Hq, Hkv, D, E, page_size,
+                       scale, window, chunk);
   else if (dtype == NHV_BF16)
     hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, dim3(blocks), dim3(256), lds, s, (const bf16_t*)q,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, (const int*)token_req,
-                       (const int*)positions, (const int*)block_tables, max_blocks, (int)n_items, Hq, Hkv, D, page_size,
-                       scale, window);
+                       (const int*)positions, (const int*)block_tables, max_blocks, (int)n_items, Hq, Hkv, D, E, page_size,
+                       scale, window, chunk);
   else
     return nhv_fail("attention: unknown dtype %d", dtype);
   NHV_LAUNCH_CHECK("paged_attention_generic");

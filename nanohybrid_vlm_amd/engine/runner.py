@@ -26,12 +26,25 @@ from ..cache.manager import NO_PAGE, CacheManager, OutOfPages, PagedGroupSpec
 from ..config.model_config import read_config_json
 from ..config.registry import resolve_architecture
 from ..native.ops import AttentionBatch
-from ..parts.base import CacheView, PagedKVNeed, StateNeed
+from ..parts.base import CacheView, CombinedNeed, PagedKVNeed, StateNeed
 from ..parts.context import GroupTables, StepContext
 from ..parts.model import DecoderModel
-from ..weights.loader import load_weights
+from ..weights.loader import checkpoint_shapes, load_weights
 
 _TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+def _paged(need) -> PagedKVNeed | None:
+    """The pages that a run-order entry needs, whether it needs only those or state beside them."""
+    if isinstance(need, CombinedNeed):
+        return need.paged
+    return need if isinstance(need, PagedKVNeed) else None
+
+
+def _state(need) -> StateNeed | None:
+    if isinstance(need, CombinedNeed):
+        return need.state
+    return need if isinstance(need, StateNeed) else None
 
 
 @dataclass
@@ -67,7 +80,8 @@ class ModelRunner:
         if model is None:
             raw = read_config_json(model_dir)
             arch = resolve_architecture(raw)
-            cfg = arch.parse_config(raw)
+            # (an architecture may take sizes that config.json does not name from the shapes of the stored tensors)
+            cfg = arch.parse_config(raw, checkpoint_shapes(model_dir)) if arch.reads_checkpoint_shapes else arch.parse_config(raw)
             # engine options that parts may care for are offered to every part's constructor
             model = DecoderModel(arch.build_spec(cfg), options={"residual_float32": bool(residual_float32)})
             load_weights(model, arch, cfg, model_dir, self.dtype, self.device)
@@ -129,17 +143,19 @@ class ModelRunner:
     # ------------------------------------------------------------------ cache
     def _make_cache(self, page_size, num_pages, num_state_slots, utilization, max_tokens):
         needs = self.model.cache_needs()
-        windows: list[int | None] = []                 # one group per distinct window
+        windows: list[tuple] = []                      # one group per distinct (window, chunk): what a query reads
         self._entry_group: dict[int, int] = {}
         for i, need in enumerate(needs):
-            if isinstance(need, PagedKVNeed):
-                if need.window not in windows:
-                    windows.append(need.window)
-                self._entry_group[i] = windows.index(need.window)
+            paged = _paged(need)
+            if paged is not None:
+                reach = (paged.window, paged.chunk)
+                if reach not in windows:
+                    windows.append(reach)
+                self._entry_group[i] = windows.index(reach)
         if not windows:
-            windows = [None]                           # a model without paged layers still has one (empty) group
+            windows = [(None, None)]                   # a model without paged layers still has one (empty) group
         self._windows = windows
-        if self.share_prefixes and any(isinstance(n, StateNeed) for n in needs):
+        if self.share_prefixes and any(_state(n) is not None for n in needs):
             # state of fixed size summarises all earlier tokens: pages alone do not bring a prefix back
             # (the reference switches the page hashes off for such models, nanovllm/config.py:384-399)
             raise ValueError("prefixes cannot be shared by a model with per-request state")
@@ -150,14 +166,14 @@ class ModelRunner:
         self._state_views: dict[int, CacheView] = {}
         self.num_state_slots = num_state_slots
         for i, need in enumerate(needs):
-            if isinstance(need, StateNeed):
+            if _state(need) is not None:
                 pool = {name: torch.zeros((num_state_slots + 1, *shape), dtype=dt, device=self.device)
-                        for name, (shape, dt) in need.tensors.items()}
+                        for name, (shape, dt) in _state(need).tensors.items()}
                 self.state_pools.append(pool)
                 self._state_views[i] = CacheView(kind="state", state=pool)
         item = torch.empty((), dtype=self.dtype).element_size()
-        page_bytes = sum(2 * page_size * n.num_kv_heads * n.head_dim * item
-                         for n in needs if isinstance(n, PagedKVNeed))
+        page_bytes = sum(page_size * n.num_kv_heads * (n.head_dim + n.value_size) * item
+                         for n in map(_paged, needs) if n is not None)
         if num_pages is None:
             num_pages = self._pages_from_free_memory(page_bytes, utilization, max_tokens)
         self._allocate_pages(num_pages)
@@ -167,22 +183,33 @@ class ModelRunner:
         needs = self.model.cache_needs()
         page_size = self.page_size
         self.num_pages = num_pages
-        groups = [PagedGroupSpec(name="all keys" if w is None else f"window {w}", page_size=page_size,
-                                 num_pages=num_pages, window=w) for w in self._windows]
+        groups = [PagedGroupSpec(name=f"window {w}" if w is not None else (f"chunk {c}" if c is not None else "all keys"),
+                                 page_size=page_size, num_pages=num_pages, window=w, chunk=c) for w, c in self._windows]
         self.cache = CacheManager(groups, self.num_state_slots, share_prefixes=self.share_prefixes)
         views: list[CacheView | None] = [None] * len(needs)
         views[:] = [self._state_views.get(i) for i in range(len(needs))]
-        self.kv_tensors: list[torch.Tensor] = []       # the pages that requests may hold, per cache unit
+        self.kv_tensors: list[torch.Tensor] = []       # the pages that requests may hold, per cache unit (keys and values apart where their head sizes differ)
         for i, need in enumerate(needs):
-            if isinstance(need, PagedKVNeed):
+            need = _paged(need)
+            if need is not None:
                 # [2, pages + 1, page_size, kv_heads, head_dim]: one token's heads lie together
                 # (nanovllm/engine/model_runner.py:870-906). The last page is handed to no request and holds zeros:
-                # the padding rows of a recorded step read their one key there.
-                kv = torch.empty((2, num_pages + 1, page_size, need.num_kv_heads, need.head_dim),
-                                 dtype=self.dtype, device=self.device)
-                kv[:, num_pages].zero_()
-                self.kv_tensors.append(kv[:, :num_pages])
-                views[i] = CacheView(kind="paged", group=self._entry_group[i], k=kv[0], v=kv[1], writes=True)
+                # the padding rows of a recorded step read their one key there. Value heads of another size than
+                # the key heads get a tensor of their own.
+                if need.value_size == need.head_dim:
+                    kv = torch.empty((2, num_pages + 1, page_size, need.num_kv_heads, need.head_dim),
+                                     dtype=self.dtype, device=self.device)
+                    kv[:, num_pages].zero_()
+                    k, v = kv[0], kv[1]
+                    self.kv_tensors.append(kv[:, :num_pages])
+                else:
+                    k = torch.empty((num_pages + 1, page_size, need.num_kv_heads, need.head_dim), dtype=self.dtype, device=self.device)
+                    v = torch.empty((num_pages + 1, page_size, need.num_kv_heads, need.value_size), dtype=self.dtype, device=self.device)
+                    k[num_pages].zero_()
+                    v[num_pages].zero_()
+                    self.kv_tensors += [k[:num_pages], v[:num_pages]]
+                state = views[i].state if views[i] is not None else None       # (a mixer that keeps pages and state)
+                views[i] = CacheView(kind="paged", group=self._entry_group[i], k=k, v=v, writes=True, state=state)
         for i, e in enumerate(self.model.run_order):
             if e.cache is not None:
                 lender = views[e.cache]
@@ -666,7 +693,7 @@ class ModelRunner:
         """Whether the next tokens of these requests can be run before the host knows them (``step_ahead``):
         a recorded graph for their number, laid out for their lengths, and a cache whose commits can be taken back."""
         if not (self.use_graphs and request_ids and len(request_ids) <= self.max_graph_batch
-                and not self.cache.share_prefixes and all(g.window is None for g in self.cache.groups)):
+                and not self.cache.share_prefixes and all(g.keeps_all for g in self.cache.groups)):
             return False
         g = self._graphs.get(next(b for b in self.graph_buckets if b >= len(request_ids)))
         if g is None or g["graph"] is None:
@@ -837,7 +864,7 @@ class ModelRunner:
             "kv_cache_bytes": sum(t.numel() * t.element_size() for t in self.kv_tensors),
             "state_pool_bytes": sum(t.numel() * t.element_size() for pool in self.state_pools for t in pool.values()),
             "page_size": self.page_size,
-            "groups": [{"name": g.name, "window": g.window, "pages": g.num_pages,
+            "groups": [{"name": g.name, "window": g.window, "chunk": g.chunk, "pages": g.num_pages,
                         "free_pages": self.cache.num_free_pages(i)} for i, g in enumerate(self.cache.groups)],
             "live_requests": len(self.cache.requests),
             "prefix_cache": {"enabled": self.cache.share_prefixes, "known_pages": len(self.cache.page_of_hash),

@@ -19,7 +19,7 @@ import torch
 from . import library
 
 CORE_SOURCES = ["error.hip", "elementwise.hip", "gemm_generic.hip", "gemm_skinny_bf16.hip", "gemm_fewrows_bf16.hip", "attention_generic.hip",
-                "sampling.hip", "measure.hip"]
+                "sampling.hip", "measure.hip", "stream_mixing.hip", "delta_rule.hip"]
 BLAS_SOURCES = ["error.hip", "gemm_library.hip"]                                                   # the vendor's matrix library, algorithm by number
 BLAS_LINK = ["-lhipblaslt"]
 ATTENTION_SOURCES = ["error.hip", "attention_decode_bf16.hip", "attention_prefill_bf16.hip"]      # compiled once per head size
@@ -175,13 +175,15 @@ class NativeBackend:
                    _ptr(q_out), _ptr(k_cache), _ptr(v_cache), qkv.shape[0], Hq, Hkv, D, int(write_kv),
                    dtype_code(qkv), wd, _stream())
 
-    def paged_attention(self, q, k_cache, v_cache, out, batch: AttentionBatch, block_tables, scale, window):
+    def paged_attention(self, q, k_cache, v_cache, out, batch: AttentionBatch, block_tables, scale, window, chunk=0):
         T, Hq, D = q.shape
         _, page_size, Hkv, _ = k_cache.shape
-        if (q.dtype == torch.bfloat16 and batch.max_q_len == 1 and D % 16 == 0 and D <= 256 and Hq // Hkv <= 16
-                and T <= 65535):
+        E = v_cache.shape[3]
+        # the kernels on the matrix cores take value heads of the key heads' size and a window or no bound at all
+        fast = q.dtype == torch.bfloat16 and E == D and not chunk and D % 16 == 0 and D <= 256
+        if fast and batch.max_q_len == 1 and Hq // Hkv <= 16 and T <= 65535:
             return self._decode_attention(q, k_cache, v_cache, out, batch, block_tables, scale, window)
-        if q.dtype == torch.bfloat16 and D % 16 == 0 and D <= 256 and batch.num_requests <= 65535 and Hkv <= 65535:
+        if fast and batch.num_requests <= 65535 and Hkv <= 65535:
             # prompt portions (and whatever single tokens share their batch) on the matrix cores
             return self._call("nhv_prefill_attention_bf16", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out),
                               _ptr(batch.cu_seqlens_q), _ptr(batch.context_lens), _ptr(block_tables),
@@ -189,7 +191,56 @@ class NativeBackend:
                               ctypes.c_float(scale), window, _stream(), lib=self.attention_lib(D))
         self._call("nhv_paged_attention_generic", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out),
                    _ptr(batch.token_req), _ptr(batch.positions), _ptr(block_tables), block_tables.shape[1], T, Hq, Hkv,
-                   D, page_size, ctypes.c_float(scale), window, dtype_code(q), _stream())
+                   D, E, page_size, ctypes.c_float(scale), window, chunk, dtype_code(q), _stream())
+
+    # -- layers that are not the pre-norm kind: norms with one number, sums over depth, rotation without a table --
+    def scalar_rmsnorm(self, x, gain, y, eps):
+        T, W = x.shape
+        self._call("nhv_scalar_rmsnorm", _ptr(x), dtype_code(x), _ptr(gain), _ptr(y), dtype_code(y), T, W,
+                   ctypes.c_float(eps), _stream())
+
+    def pair_norm_mean(self, a, wa, b, wb, y, eps):
+        T, W = a.shape
+        self._call("nhv_pair_norm_mean", _ptr(a), _ptr(wa), _ptr(b), _ptr(wb), _ptr(y), T, W, ctypes.c_float(eps),
+                   dtype_code(a), _stream())
+
+    def depth_mix(self, x, a, b, results, index, weights, out, gain, normed, eps):
+        T, W = x.shape
+        self._call("nhv_depth_mix", _ptr(x), _ptr(a), _ptr(b), _ptr(results), ctypes.c_longlong(results.stride(0)), index,
+                   _ptr(weights), _ptr(out), _ptr(gain), _ptr(normed), T, W, ctypes.c_float(eps), dtype_code(a), _stream())
+
+    def rotary_split_write(self, qkv, bias, qk_freqs, rot, v_freqs, positions, slot_mapping, q_out, k_cache, v_cache,
+                           Hq, Hkv, D, E, with_kv):
+        self._call("nhv_rotary_split_write", _ptr(qkv), _ptr(bias), _ptr(qk_freqs), rot, _ptr(v_freqs), _ptr(positions),
+                   _ptr(slot_mapping), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), qkv.shape[0], Hq, Hkv, D, E,
+                   int(with_kv), dtype_code(qkv), _stream())
+
+    def turn_back(self, x, freqs, positions):
+        T, H, E = x.shape
+        self._call("nhv_turn_back", _ptr(x), _ptr(freqs), _ptr(positions), T, H, E, dtype_code(x), _stream())
+
+    # -- the gated delta rule --
+    def delta_prepare(self, proj, taps, kept, a_lin, dt_bias, a_log, batch, state_slots, q, k, v, beta, H, G, D, E):
+        self._call("nhv_delta_prepare", _ptr(proj), dtype_code(proj), _ptr(taps), taps.shape[1], _ptr(kept), _ptr(a_lin),
+                   _ptr(dt_bias), _ptr(a_log), _ptr(batch.token_req), _ptr(batch.positions), _ptr(batch.cu_seqlens_q),
+                   _ptr(state_slots), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), proj.shape[0], H, G, D, E, _stream())
+
+    def conv_state_update(self, proj, kept, n_taps, batch, state_slots, channels):
+        self._call("nhv_conv_state_update", _ptr(proj), dtype_code(proj), proj.shape[1], _ptr(kept), n_taps,
+                   _ptr(batch.positions), _ptr(batch.cu_seqlens_q), _ptr(state_slots), batch.num_requests, channels,
+                   _stream())
+
+    def delta_rule(self, q, k, v, decay, beta, state, out, batch, state_slots):
+        T, G, D = q.shape
+        _, H, E = v.shape
+        self._call("nhv_delta_rule", _ptr(q), _ptr(k), _ptr(v), _ptr(decay), _ptr(beta), _ptr(state), _ptr(out),
+                   _ptr(batch.positions), _ptr(batch.cu_seqlens_q), _ptr(state_slots), batch.num_requests, H, G, D, E,
+                   _stream())
+
+    def gated_head_norm(self, o, gate, w, y, eps):
+        T, H, E = o.shape
+        self._call("nhv_gated_head_norm", _ptr(o), _ptr(gate), _ptr(w), _ptr(y), T, H, E, ctypes.c_float(eps),
+                   dtype_code(y), _stream())
 
     def _decode_attention(self, q, k_cache, v_cache, out, batch, block_tables, scale, window):
         """Single tokens in bfloat16: keys split over waves, then merged."""
@@ -836,14 +887,21 @@ def qk_rope_write(qkv, bias, q_norm_w, k_norm_w, eps, cos_sin, positions, slot_m
 
 
 def paged_attention(q, k_cache, v_cache, batch: AttentionBatch, block_tables, scale: float,
-                    window: int | None = None) -> torch.Tensor:
+                    window: int | None = None, chunk: int | None = None) -> torch.Tensor:
+    """Every query reads its request's keys up to its own position: all of them, the last ``window``, or (``chunk``)
+    those of its own block of ``chunk`` positions counted from the request's start. The value heads may have another
+    size than the key heads: the result is [tokens, heads, value size]."""
     _need(q.dim() == 3, "attention: q must be [tokens, heads, head_dim]")
     T, Hq, D = q.shape
     _dense(q, "attention: q")
     dtype_code(q)
     _need(k_cache.dim() == 4 and k_cache.shape[3] == D, lambda: f"attention: cache shape {tuple(k_cache.shape)} with head size {D}")
     _dense(k_cache, "attention: k_cache", dtype=q.dtype)
-    _dense(v_cache, "attention: v_cache", tuple(k_cache.shape), q.dtype)
+    _need(v_cache.dim() == 4 and tuple(v_cache.shape[:3]) == tuple(k_cache.shape[:3]),
+          lambda: f"attention: value cache {tuple(v_cache.shape)} beside key cache {tuple(k_cache.shape)}")
+    _dense(v_cache, "attention: v_cache", dtype=q.dtype)
+    _need(not (window and chunk), "attention: a window or a chunk, not both")
+    _need(chunk is None or chunk > 0, lambda: f"attention: chunk {chunk}")
     Hkv = k_cache.shape[2]
     _need(Hq % Hkv == 0, lambda: f"attention: {Hq} query heads are not a multiple of {Hkv} key heads")
     _need(T == batch.num_tokens, lambda: f"attention: {T} tokens but the batch has {batch.num_tokens}")
@@ -856,8 +914,11 @@ def paged_attention(q, k_cache, v_cache, batch: AttentionBatch, block_tables, sc
     _need(block_tables.shape[1] * page_size >= batch.max_context_len,
           lambda: f"attention: block tables of {block_tables.shape[1]} pages of {page_size} are too short for "
           f"{batch.max_context_len} keys")
-    out = torch.empty_like(q)
-    backend().paged_attention(q, k_cache, v_cache, out, batch, block_tables, float(scale), int(window or 0))
+    out = torch.empty((T, Hq, v_cache.shape[3]), dtype=q.dtype, device=q.device)
+    if chunk:
+        backend().paged_attention(q, k_cache, v_cache, out, batch, block_tables, float(scale), 0, int(chunk))
+    else:
+        backend().paged_attention(q, k_cache, v_cache, out, batch, block_tables, float(scale), int(window or 0))
     return out
 
 
@@ -927,6 +988,170 @@ def gated_linear(x, w: torch.Tensor) -> torch.Tensor:
         if fused(x, w, out):
             return out
     return silu_mul(linear(x, w))
+
+
+# ------------------------------------------------------------------ layers that are not the pre-norm kind
+def _float_vector(t: torch.Tensor, name: str, shape: tuple) -> None:
+    _dense(t, name, shape, torch.float32)
+
+
+def scalar_rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out_dtype=None) -> torch.Tensor:
+    """x / sqrt(mean(x^2) + eps) * gain, ``gain`` one float32 number on the device. ``x`` and the result may differ
+    in element type (a float32 stream normed into bfloat16 rows, bfloat16 rows normed into a float32 stream)."""
+    _need(x.dim() == 2, "scalar_rmsnorm: x must be [tokens, width]")
+    _dense(x, "scalar_rmsnorm: x")
+    _need(gain.numel() == 1, lambda: f"scalar_rmsnorm: the weight is one number, got {tuple(gain.shape)}")
+    _dense(gain, "scalar_rmsnorm: weight", dtype=torch.float32)
+    dtype_code(x)
+    y = torch.empty(x.shape, dtype=out_dtype or x.dtype, device=x.device)
+    dtype_code(y)
+    if x.shape[0]:
+        backend().scalar_rmsnorm(x, gain, y, float(eps))
+    return y
+
+
+def pair_norm_mean(a: torch.Tensor, wa: torch.Tensor, b: torch.Tensor, wb: torch.Tensor, eps: float) -> torch.Tensor:
+    """(norm(a) * wa + norm(b) * wb) / 2 row by row, norm = x / sqrt(mean(x^2) + eps); float32 weights."""
+    _need(a.dim() == 2, "pair_norm_mean: rows must be [tokens, width]")
+    _dense(a, "pair_norm_mean: a")
+    _dense(b, "pair_norm_mean: b", tuple(a.shape), a.dtype)
+    _float_vector(wa, "pair_norm_mean: first weight", (a.shape[1],))
+    _float_vector(wb, "pair_norm_mean: second weight", (a.shape[1],))
+    dtype_code(a)
+    y = torch.empty_like(a)
+    backend().pair_norm_mean(a, wa, b, wb, y, float(eps))
+    return y
+
+
+def depth_mix(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor | None, results: torch.Tensor, index: int,
+              weights: torch.Tensor, gain: torch.Tensor | None = None, eps: float = 0.0):
+    """results[index + 1] = x + (a + b) (and results[0] = x when ``index`` is 0); returns the float32 stream
+    sum over j <= index + 1 of weights[j] * results[j], and with ``gain`` also its RMS norm (one number as weight)
+    in the element type of ``a``. ``x``: [tokens, width] float32; ``results``: [depth, tokens, width] float32."""
+    _need(x.dim() == 2, "depth_mix: x must be [tokens, width]")
+    T, W = x.shape
+    _dense(x, "depth_mix: x", dtype=torch.float32)
+    _dense(a, "depth_mix: a", (T, W))
+    dtype_code(a)
+    if b is not None:
+        _dense(b, "depth_mix: b", (T, W), a.dtype)
+    _need(results.dim() == 3 and tuple(results.shape[1:]) == (T, W) and 0 <= index and index + 2 <= results.shape[0],
+          lambda: f"depth_mix: results {tuple(results.shape)} for index {index} and rows {(T, W)}")
+    _dense(results, "depth_mix: results", dtype=torch.float32)
+    _float_vector(weights, "depth_mix: weights", (index + 2,))
+    out = torch.empty_like(x)
+    normed = None
+    if gain is not None:
+        _need(gain.numel() == 1, "depth_mix: the norm's weight is one number")
+        _dense(gain, "depth_mix: norm weight", dtype=torch.float32)
+        normed = torch.empty((T, W), dtype=a.dtype, device=a.device)
+    backend().depth_mix(x, a, b, results, int(index), weights, out, gain, normed, float(eps))
+    return (out, normed) if gain is not None else out
+
+
+def rotary_split_write(qkv: torch.Tensor, bias: torch.Tensor | None, qk_freqs: torch.Tensor | None,
+                       v_freqs: torch.Tensor | None, positions: torch.Tensor, slot_mapping, k_cache, v_cache,
+                       num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, with_kv: bool = True) -> torch.Tensor:
+    """Splits the packed projection q | k | v (``with_kv``) or q alone, adds the bias, turns pair (i, i + r) of every
+    query and key head by position * qk_freqs[i] (r = len(qk_freqs); the coordinates from 2 r on pass), turns the
+    value heads the same way over all their coordinates if ``v_freqs`` is given, stores keys and values at the
+    step's slots and returns q as [tokens, heads, head_dim]. Angles are taken in float from the position: no table."""
+    T = qkv.shape[0]
+    width = num_heads * head_dim + (num_kv_heads * (head_dim + value_dim) if with_kv else 0)
+    _dense(qkv, "rotary_split_write: qkv", (T, width))
+    dtype_code(qkv)
+    if bias is not None:
+        _dense(bias, "rotary_split_write: bias", (width,), qkv.dtype)
+    rot = 0
+    if qk_freqs is not None:
+        rot = 2 * qk_freqs.shape[0]
+        _need(rot <= head_dim, lambda: f"rotary_split_write: rotary size {rot} with head size {head_dim}")
+        _float_vector(qk_freqs, "rotary_split_write: frequencies", (rot // 2,))
+    _dense(positions, "rotary_split_write: positions", (T,), torch.int32)
+    if with_kv:
+        _dense(slot_mapping, "rotary_split_write: slot_mapping", (T,), torch.int32)
+        _need(k_cache.dim() == 4 and tuple(k_cache.shape[2:]) == (num_kv_heads, head_dim),
+              lambda: f"rotary_split_write: key cache {tuple(k_cache.shape)} does not fit {num_kv_heads} heads of {head_dim}")
+        _need(v_cache.dim() == 4 and tuple(v_cache.shape[2:]) == (num_kv_heads, value_dim),
+              lambda: f"rotary_split_write: value cache {tuple(v_cache.shape)} does not fit {num_kv_heads} heads of {value_dim}")
+        _dense(k_cache, "rotary_split_write: k_cache", dtype=qkv.dtype)
+        _dense(v_cache, "rotary_split_write: v_cache", dtype=qkv.dtype)
+        if v_freqs is not None:
+            _need(value_dim % 2 == 0, "rotary_split_write: value heads of odd size cannot be turned")
+            _float_vector(v_freqs, "rotary_split_write: value frequencies", (value_dim // 2,))
+    q_out = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    if T:
+        backend().rotary_split_write(qkv, bias, qk_freqs, rot, v_freqs if with_kv else None, positions,
+                                     slot_mapping if with_kv else None, q_out, k_cache if with_kv else None,
+                                     v_cache if with_kv else None, num_heads, num_kv_heads, head_dim, value_dim, with_kv)
+    return q_out
+
+
+def turn_back_(x: torch.Tensor, freqs: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+    """x[tokens, heads, size] in place: pair (m, m + size / 2) of every head turns by -position * freqs[m]."""
+    _need(x.dim() == 3 and x.shape[2] % 2 == 0, "turn_back: x must be [tokens, heads, even size]")
+    _dense(x, "turn_back: x")
+    dtype_code(x)
+    _float_vector(freqs, "turn_back: frequencies", (x.shape[2] // 2,))
+    _dense(positions, "turn_back: positions", (x.shape[0],), torch.int32)
+    if x.shape[0]:
+        backend().turn_back(x, freqs, positions)
+    return x
+
+
+def gated_delta_rule(proj: torch.Tensor, a_lin: torch.Tensor, gate_lin: torch.Tensor, taps: torch.Tensor,
+                     dt_bias: torch.Tensor, a_log: torch.Tensor, norm_weight: torch.Tensor, eps: float,
+                     kept: torch.Tensor, state: torch.Tensor, batch: AttentionBatch, state_slots: torch.Tensor,
+                     num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, out_dtype) -> torch.Tensor:
+    """The recurrent mixer between its projections: short causal convolutions and SiLU on q, k, v (``proj``:
+    [tokens, q | k | v | beta] as projected; ``taps`` [channels, n]; ``kept`` [slots, channels, n - 1], a request's
+    last inputs, updated here), unit length for q and k per head, beta = sigmoid, the decays
+    exp(-exp(a_log) softplus(a_lin + dt_bias)) per head and key channel, the recurrence over every request's tokens in
+    order from and into ``state`` [slots, heads, value_dim, head_dim] (a request whose first token is at position 0
+    starts from zero), then per head the read-out over its root mean square times ``norm_weight`` times
+    sigmoid(gate_lin). Returns [tokens, heads * value_dim] in ``out_dtype``. ``a_lin`` is overwritten."""
+    T = proj.shape[0]
+    H, G, D, E = num_heads, num_kv_heads, head_dim, value_dim
+    C = 2 * G * D + H * E
+    _need(H % G == 0, lambda: f"gated_delta_rule: {H} heads are not a multiple of {G} key heads")
+    _dense(proj, "gated_delta_rule: proj", (T, C + H))
+    dtype_code(proj)
+    _float_vector(a_lin, "gated_delta_rule: decays' linear part", (T, H * D))
+    _float_vector(gate_lin, "gated_delta_rule: gates' linear part", (T, H * E))
+    _need(taps.dim() == 2 and taps.shape[0] == C and 1 <= taps.shape[1] <= 16,
+          lambda: f"gated_delta_rule: taps {tuple(taps.shape)} for {C} channels (1 to 16 taps)")
+    _dense(taps, "gated_delta_rule: taps", dtype=torch.float32)
+    n = taps.shape[1]
+    _float_vector(dt_bias, "gated_delta_rule: dt_bias", (H * D,))
+    _float_vector(a_log, "gated_delta_rule: a_log", (H,))
+    _float_vector(norm_weight, "gated_delta_rule: norm weight", (E,))
+    _need(kept.dim() == 3 and tuple(kept.shape[1:]) == (C, n - 1), lambda: f"gated_delta_rule: kept inputs {tuple(kept.shape)}")
+    _dense(kept, "gated_delta_rule: kept inputs", dtype=torch.float32)
+    _need(state.dim() == 4 and tuple(state.shape[1:]) == (H, E, D) and state.shape[0] == kept.shape[0],
+          lambda: f"gated_delta_rule: state {tuple(state.shape)}")
+    _dense(state, "gated_delta_rule: state", dtype=torch.float32)
+    B = batch.num_requests
+    _need(T == batch.num_tokens, lambda: f"gated_delta_rule: {T} tokens but the batch has {batch.num_tokens}")
+    _dense(batch.token_req, "gated_delta_rule: token_req", (T,), torch.int32)
+    _dense(batch.positions, "gated_delta_rule: positions", (T,), torch.int32)
+    _dense(batch.cu_seqlens_q, "gated_delta_rule: cu_seqlens_q", (B + 1,), torch.int32)
+    _dense(state_slots, "gated_delta_rule: state_slots", (B,), torch.int32)
+    dev = proj.device
+    q = torch.empty((T, G, D), dtype=torch.float32, device=dev)
+    k = torch.empty((T, G, D), dtype=torch.float32, device=dev)
+    v = torch.empty((T, H, E), dtype=torch.float32, device=dev)
+    beta = torch.empty((T, H), dtype=torch.float32, device=dev)
+    o = torch.empty((T, H, E), dtype=torch.float32, device=dev)
+    y = torch.empty((T, H * E), dtype=out_dtype, device=dev)
+    dtype_code(y)
+    if T == 0:
+        return y
+    b = backend()
+    b.delta_prepare(proj, taps, kept, a_lin, dt_bias, a_log, batch, state_slots, q, k, v, beta, H, G, D, E)
+    b.conv_state_update(proj, kept, n, batch, state_slots, C)
+    b.delta_rule(q, k, v, a_lin.view(T, H, D), beta, state, o, batch, state_slots)
+    b.gated_head_norm(o, gate_lin.view(T, H, E), norm_weight, y.view(T, H, E), float(eps))
+    return y
 
 
 def sample(logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:

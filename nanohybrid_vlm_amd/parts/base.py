@@ -21,6 +21,9 @@ class ParamSpec:
     shape: tuple[int, ...]
     init: str = "normal"          # random-weights mode: "normal" N(0, 0.02^2), "norm" 1 + N(0, 0.1^2), "zeros"
     keeps_float32: bool = False   # a tensor stored in 32-bit stays so even in a bfloat16 run
+    always_float32: bool = False  # the parameter is float32 whatever the file stores and the run computes in
+    init_mean: float | None = None   # random-weights mode: N(init_mean, init_std^2) in place of what ``init`` names
+    init_std: float | None = None
 
 
 @dataclass(frozen=True)
@@ -30,6 +33,20 @@ class PagedKVNeed:
     num_kv_heads: int
     head_dim: int
     window: int | None = None     # None: all keys; n: only the last n are read
+    value_dim: int | None = None  # size of a value head where it is not ``head_dim``
+    chunk: int | None = None      # n: a query reads only the keys of its own block of n positions (counted from 0)
+
+    @property
+    def value_size(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
+
+
+@dataclass(frozen=True)
+class CombinedNeed:
+    """A mixer that is several mixers side by side: at most one paged need and one state need among them."""
+
+    paged: PagedKVNeed | None = None
+    state: "StateNeed | None" = None
 
 
 @dataclass(frozen=True)

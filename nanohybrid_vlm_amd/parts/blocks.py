@@ -1,7 +1,10 @@
 """How a layer's norm, mixer and feed-forward are arranged."""
 from __future__ import annotations
 
-from .base import BLOCKS, Part
+import torch
+
+from ..native import ops
+from .base import BLOCKS, ParamSpec, Part
 
 
 @BLOCKS.register("prenorm")
@@ -60,3 +63,47 @@ def _add_to(part, norm, residual, reader) -> dict:
     if norm is not None and getattr(part, "adds_to_residual", False) and getattr(norm, "takes_summed", False):
         return {"add_to": norm.add_to(residual, reader if getattr(reader, "takes_deferred_norm", False) else None)}
     return {}
+
+
+@BLOCKS.register("parallel_depth_mix")
+class ParallelDepthMixBlock(Part):
+    """One norm, mixer and feed-forward side by side on its output, and a weighted sum over depth:
+        h = norm(x);  X_(i+1) = x + (mixer(h) + feed_forward(h));  x <- sum over j <= i + 1 of w[j] X_j,
+    where X_0 is the stream that entered the first such block and i = ``depth_index`` counts the blocks before this
+    one. The stream is float32 and is what the block takes and returns as ``hidden`` (there is no residual beside
+    it); the results X_j of a step live in ``step.scratch`` ([``depth_total`` + 1, tokens, width] float32). The
+    feed-forward may be absent."""
+
+    norm_slots = ("norm",)
+
+    def __init__(self, mixer, feed_forward, norm, depth_index: int, depth_total: int):
+        if not 0 <= depth_index < depth_total:
+            raise ValueError(f"block {depth_index} of {depth_total}")
+        self.mixer, self.feed_forward, self.norm = mixer, feed_forward, norm
+        self.depth_index, self.depth_total = depth_index, depth_total
+        self.row_dtype = None
+
+    def children(self):
+        out = {"norm": self.norm, "mixer": self.mixer}
+        if self.feed_forward is not None:
+            out["feed_forward"] = self.feed_forward
+        return out
+
+    def param_specs(self):
+        n = self.depth_index + 2
+        return {"depth.weight": ParamSpec((n,), always_float32=True, init_mean=1.0 / n, init_std=0.3 / n)}
+
+    def forward(self, hidden, residual, step, cache):
+        if residual is not None:
+            raise ValueError("this block carries its stream itself and takes no residual beside it")
+        if hidden.dtype != torch.float32:
+            hidden = hidden.float()
+        T, W = hidden.shape
+        results = step.scratch.get("depth_results")
+        if results is None or self.depth_index == 0:
+            results = step.scratch["depth_results"] = torch.empty((self.depth_total + 1, T, W), dtype=torch.float32,
+                                                                   device=hidden.device)
+        h = self.norm.forward(hidden, out_dtype=self.row_dtype or torch.float32)
+        mixed = self.mixer.forward(h, step, cache)
+        fed = self.feed_forward.forward(h, step) if self.feed_forward is not None else None
+        return ops.depth_mix(hidden, mixed, fed, results, self.depth_index, self.depth_weight), None

@@ -32,3 +32,4 @@ class StepContext:
     logit_rows: torch.Tensor | None  # [n] int32: the tokens whose logits are wanted
     num_logit_rows: int = 0
     host: dict = field(default_factory=dict)   # the same facts as Python lists, for parts that work on the host
+    scratch: dict = field(default_factory=dict)   # device buffers that parts of one step share (made by the first that needs them)

@@ -1,11 +1,13 @@
 """Token mixers. ``GQAAttention`` follows nanovllm/models/qwen3.py:14-88 and
-nanovllm/layers/attention.py:43-75."""
+nanovllm/layers/attention.py:43-75. ``RotaryAttention`` is softmax attention in a more general make (value heads of
+their own size, biases, a chunk mask, turned values, keys and values lent by another layer), ``GatedDeltaRule`` a
+recurrent mixer with a matrix of state per head, ``NormedPair`` two mixers side by side."""
 from __future__ import annotations
 
 import torch
 
 from ..native import ops
-from .base import MIXERS, CacheView, PagedKVNeed, ParamSpec, Part
+from .base import MIXERS, CacheView, CombinedNeed, PagedKVNeed, ParamSpec, Part, StateNeed
 
 
 @MIXERS.register("gqa_attention")
@@ -78,3 +80,161 @@ class GQAAttention(Part):
             write_kv=cache.writes, pair_axes=pair_axes)
         o = ops.paged_attention(q, cache.k, cache.v, step.attention, tables.block_tables, self.scale, self.window)
         return ops.linear(o.view(o.shape[0], self.num_heads * self.head_dim), self.o_weight, add_to=add_to)
+
+
+@MIXERS.register("rotary_attention")
+class RotaryAttention(Part):
+    """Softmax attention with grouped key/value heads over the paged cache, in a more general make than
+    ``GQAAttention``: value heads of a size of their own (``value_dim``), optional biases on q, k and v, the rotation
+    given by frequencies (``position``: a ``rotary_frequencies`` encoding; angles are taken from the position, no
+    table), and which keys a query at position i reads: all j <= i, the last ``window`` of them, or (``chunk`` = n)
+    those with floor(j / n) = floor(i / n), blocks counted from the start of the request. ``rotate_values``: the
+    value at position j is stored turned by j over all its coordinates (pairs (m, m + value_dim / 2), frequencies of
+    the encoding's base over value_dim, unscaled), and each head's result at position i is turned back by i.
+    ``own_kv`` False: the layer has no key and value projections and reads the cache of the run-order entry it
+    borrows from (keys as stored, after rotation) with queries, mask and output projection of its own."""
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float,
+                 bias: bool, position, chunk: int | None = None, window: int | None = None, rotate_values: bool = False,
+                 own_kv: bool = True):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} key/value heads")
+        if window and chunk:
+            raise ValueError("a window or a chunk, not both")
+        if rotate_values and value_dim % 2:
+            raise ValueError(f"values of odd size {value_dim} cannot be turned")
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.head_dim, self.value_dim, self.scale, self.bias = head_dim, value_dim, scale, bias
+        self.position, self.chunk, self.window = position, chunk or None, window or None
+        self.rotate_values, self.own_kv = rotate_values, own_kv
+        self.qkv_weight = self.qkv_bias = self.o_weight = None
+
+    def _packed_width(self) -> int:
+        width = self.num_heads * self.head_dim
+        if self.own_kv:
+            width += self.num_kv_heads * (self.head_dim + self.value_dim)
+        return width
+
+    def param_specs(self):
+        specs = {"qkv.weight": ParamSpec((self._packed_width(), self.hidden_size)),
+                 "o.weight": ParamSpec((self.hidden_size, self.num_heads * self.value_dim))}
+        if self.bias:
+            specs["qkv.bias"] = ParamSpec((self._packed_width(),), init="zeros")
+        return specs
+
+    def bind(self, params):
+        self.qkv_weight, self.o_weight = params["qkv.weight"], params["o.weight"]
+        self.qkv_bias = params.get("qkv.bias")
+
+    def cache_need(self):
+        return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window,
+                           None if self.value_dim == self.head_dim else self.value_dim, self.chunk)
+
+    def forward(self, x, step, cache: CacheView):
+        tables = step.groups[cache.group]
+        writes = self.own_kv and cache.writes
+        if not self.own_kv and cache.writes:
+            raise ValueError("an attention layer without key and value projections must borrow another entry's cache")
+        qkv = ops.linear(x, self.qkv_weight)
+        if self.own_kv and not writes:               # a layer with projections of its own that reads a lent cache
+            qkv = qkv[:, :self.num_heads * self.head_dim].contiguous()
+        bias = self.qkv_bias if (self.qkv_bias is None or writes or not self.own_kv) else \
+            self.qkv_bias[:self.num_heads * self.head_dim].contiguous()
+        freqs = self.position.frequencies() if self.position is not None and self.position.rotary_dim else None
+        v_freqs = self.position.frequencies_for(self.value_dim) if self.rotate_values else None
+        q = ops.rotary_split_write(qkv, bias, freqs, v_freqs, step.token_positions, tables.slot_mapping, cache.k, cache.v,
+                                   self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, with_kv=writes)
+        o = ops.paged_attention(q, cache.k, cache.v, step.attention, tables.block_tables, self.scale, self.window, self.chunk)
+        if self.rotate_values:
+            ops.turn_back_(o, v_freqs, step.token_positions)
+        return ops.linear(o.view(o.shape[0], self.num_heads * self.value_dim), self.o_weight)
+
+
+@MIXERS.register("gated_delta_rule")
+class GatedDeltaRule(Part):
+    """A recurrent mixer: per head a matrix S[head_dim, value_dim] of float32 state per request,
+        S <- diag(g_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
+    (the read-out sees the token's own write). q, k (``num_kv_heads`` heads of ``head_dim``; head h of the
+    ``num_heads`` value heads uses q/k head h // (num_heads / num_kv_heads)) and v pass a causal convolution over
+    time of ``conv_taps`` taps per channel and SiLU; q and k are made unit vectors per head (1e-6 under the root),
+    q also times head_dim^(-1/2); beta = sigmoid(W_b x); g = exp(-exp(A_log_h) softplus(W_a2 W_a1 x + dt_bias)) per
+    head and key channel; the read-out is divided by its root mean square per head (``eps``), multiplied by a weight
+    over value_dim and by sigmoid(W_g2 W_g1 x), and projected. The state and the last taps - 1 inputs of the
+    convolutions live in the request's state slot; a request that starts at position 0 starts from zeros.
+    ``decay_rank``, ``gate_rank``: the inner sizes of the two low-rank projections."""
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, conv_taps: int,
+                 decay_rank: int, gate_rank: int, eps: float, position=None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} key heads")
+        if not 1 <= conv_taps <= 16:
+            raise ValueError(f"1 to 16 taps are taken, got {conv_taps}")
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.head_dim, self.value_dim, self.conv_taps = head_dim, value_dim, conv_taps
+        self.decay_rank, self.gate_rank, self.eps = decay_rank, gate_rank, eps
+        self.channels = 2 * num_kv_heads * head_dim + num_heads * value_dim
+
+    def param_specs(self):
+        H, D, E, W = self.num_heads, self.head_dim, self.value_dim, self.hidden_size
+        return {
+            "in.weight": ParamSpec((self.channels + H, W)),                  # q | k | v | beta
+            "conv.weight": ParamSpec((self.channels, self.conv_taps), always_float32=True, init_mean=0.0, init_std=0.5),
+            "a1.weight": ParamSpec((self.decay_rank, W)),
+            "a2.weight": ParamSpec((H * D, self.decay_rank)),
+            "dt_bias": ParamSpec((H * D,), always_float32=True, init_mean=-1.0, init_std=1.0),
+            "A_log": ParamSpec((H,), always_float32=True, init_mean=-1.0, init_std=0.5),
+            "g1.weight": ParamSpec((self.gate_rank, W)),
+            "g2.weight": ParamSpec((H * E, self.gate_rank)),
+            "norm.weight": ParamSpec((E,), init="norm", always_float32=True),
+            "o.weight": ParamSpec((W, H * E)),
+        }
+
+    def cache_need(self):
+        return StateNeed({"S": ((self.num_heads, self.value_dim, self.head_dim), torch.float32),
+                          "kept": ((self.channels, self.conv_taps - 1), torch.float32)})
+
+    def forward(self, x, step, cache: CacheView):
+        proj = ops.linear(x, self.in_weight, out_dtype=torch.float32)
+        a_lin = ops.linear(ops.linear(x, self.a1_weight), self.a2_weight, out_dtype=torch.float32)
+        g_lin = ops.linear(ops.linear(x, self.g1_weight), self.g2_weight, out_dtype=torch.float32)
+        y = ops.gated_delta_rule(proj, a_lin, g_lin, self.conv_weight, self.dt_bias, self.A_log, self.norm_weight, self.eps,
+                                 cache.state["kept"], cache.state["S"], step.attention, step.state_slots, self.num_heads,
+                                 self.num_kv_heads, self.head_dim, self.value_dim, x.dtype)
+        return ops.linear(y, self.o_weight)
+
+
+@MIXERS.register("normed_pair")
+class NormedPair(Part):
+    """Two mixers side by side that read the same rows: half the sum of their results, each first RMS-normed over
+    the width (``eps``) with a plain weight vector of its own. One of them may keep pages and the other state."""
+
+    def __init__(self, hidden_size: int, left: dict, right: dict, eps: float, position=None, **offered):
+        self.hidden_size, self.eps = hidden_size, eps
+        self.left = MIXERS.build(left, offered=offered, position=position)
+        self.right = MIXERS.build(right, offered=offered, position=position)
+        self.recordable = self.left.recordable and self.right.recordable
+
+    def children(self):
+        return {"left": self.left, "right": self.right}
+
+    def param_specs(self):
+        return {"left_out.weight": ParamSpec((self.hidden_size,), init="norm", always_float32=True),
+                "right_out.weight": ParamSpec((self.hidden_size,), init="norm", always_float32=True)}
+
+    def cache_need(self):
+        paged = state = None
+        for need in (self.left.cache_need(), self.right.cache_need()):
+            if isinstance(need, PagedKVNeed):
+                if paged is not None:
+                    raise ValueError("two mixers side by side cannot both keep pages")
+                paged = need
+            elif isinstance(need, StateNeed):
+                if state is not None:
+                    raise ValueError("two mixers side by side cannot both keep state")
+                state = need
+        return CombinedNeed(paged, state)
+
+    def forward(self, x, step, cache: CacheView):
+        a = self.left.forward(x, step, cache)
+        b = self.right.forward(x, step, cache)
+        return ops.pair_norm_mean(a, self.left_out_weight, b, self.right_out_weight, self.eps)

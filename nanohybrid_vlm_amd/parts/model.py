@@ -12,8 +12,10 @@ from dataclasses import dataclass, field
 import torch
 
 from ..native import ops
-from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheView, PagedKVNeed, ParamSpec, Part,
-                   StateNeed)
+from dataclasses import replace
+
+from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheView, CombinedNeed, PagedKVNeed, ParamSpec,
+                   Part, StateNeed)
 
 
 @dataclass
@@ -25,7 +27,7 @@ class LayerSpec:
     ``norms[slot]`` if the layer names that slot, else from ``norm``."""
 
     mixer: dict
-    feed_forward: dict
+    feed_forward: dict | None             # None: the layer has no feed-forward (its block must take that)
     norm: dict | None = None              # the norm of every slot that ``norms`` does not name
     block: dict = field(default_factory=lambda: {"kind": "prenorm"})
     position: str | None = "default"      # name in ModelSpec.positions that the mixer gets, or None
@@ -62,6 +64,7 @@ class ModelSpec:
     embed_scale: float | None = None          # the embedding's rows are multiplied by this (in float, then rounded)
     logit_cap: float | None = None            # logits become cap * tanh(logits / cap)
     position_axes: int = 1                    # coordinates of a token's position (a step carries [axes, tokens])
+    embed_norm: dict | None = None            # a norm that the embedding's rows pass before the first layer
 
     def order(self) -> list[RunEntry]:
         if self.run_order is None:
@@ -87,7 +90,7 @@ class DecoderModel(Part):
             if ls.position is not None:
                 mixer_args["position"] = self.positions[ls.position]
             mixer = MIXERS.build(ls.mixer, offered=options, **mixer_args)
-            ff = FEED_FORWARDS.build(ls.feed_forward, offered=options)
+            ff = FEED_FORWARDS.build(ls.feed_forward, offered=options) if ls.feed_forward is not None else None
             # the block says which norms it takes; the layer says what each of them is
             slots = getattr(BLOCKS.maker(ls.block.get("kind")), "norm_slots", ())
             norms = {slot: NORMS.build(ls.norm_spec(slot), offered=options) for slot in slots}
@@ -97,6 +100,7 @@ class DecoderModel(Part):
                                  f"slots {list(slots)}")
             self.layers.append(BLOCKS.build(ls.block, offered=options, mixer=mixer, feed_forward=ff, **norms))
         self.final_norm = NORMS.build(spec.final_norm, offered=options)
+        self.embed_norm = NORMS.build(spec.embed_norm, offered=options) if spec.embed_norm is not None else None
         self.run_order = spec.order()
         for i, e in enumerate(self.run_order):
             if not 0 <= e.layer < len(self.layers):
@@ -105,7 +109,13 @@ class DecoderModel(Part):
                 if not 0 <= e.cache < i or self.run_order[e.cache].cache is not None:
                     raise ValueError(f"run order entry {i} reads the cache of entry {e.cache}, which must be an "
                                      f"earlier entry with a cache of its own")
-                if self.layers[e.layer].mixer.cache_need() != self.layers[self.run_order[e.cache].layer].mixer.cache_need():
+                mine = self.layers[e.layer].mixer.cache_need()
+                lent = self.layers[self.run_order[e.cache].layer].mixer.cache_need()
+                if isinstance(mine, PagedKVNeed) and isinstance(lent, PagedKVNeed):
+                    # the same pages serve both if what a page holds is the same; the blocks of positions that
+                    # each reads may differ in size (the pages are then kept for all keys)
+                    mine, lent = replace(mine, chunk=None), replace(lent, chunk=None)
+                if mine != lent:
                     raise ValueError(f"run order entry {i} and entry {e.cache} need different caches")
         self.embed_weight = None
         self.head_weight = None
@@ -122,12 +132,17 @@ class DecoderModel(Part):
     def children(self):
         out = {f"layers.{i}": layer for i, layer in enumerate(self.layers)}
         out["final_norm"] = self.final_norm
+        if self.embed_norm is not None:
+            out["embed_norm"] = self.embed_norm
         return out
 
     def bind(self, params):
         self.embed_weight = params["embed.weight"]
         # tied: the head reads the embedding's own storage (nanovllm/models/qwen3.py:202-203)
         self.head_weight = params["embed.weight"] if self.spec.tie_embeddings else params["head.weight"]
+        # every part may ask which element type the model's rows have (parts that take or give a float32 stream)
+        for part in self.walk():
+            part.row_dtype = self.embed_weight.dtype
 
     def to(self, device):
         for p in self.positions.values():
@@ -147,6 +162,13 @@ class DecoderModel(Part):
         out = []
         for e in self.run_order:
             out.append(self.layers[e.layer].mixer.cache_need() if e.cache is None else None)
+        # pages that another entry reads as well are kept for the reader whose mask reaches furthest back: where the
+        # readers' masks differ, all keys are kept
+        for i, e in enumerate(self.run_order):
+            if e.cache is not None and isinstance(out[e.cache], PagedKVNeed):
+                mine, lent = self.layers[e.layer].mixer.cache_need(), out[e.cache]
+                if mine.chunk != lent.chunk:
+                    out[e.cache] = replace(lent, chunk=None)
         return out
 
     def attach_cache(self, views: list[CacheView]) -> None:
@@ -159,6 +181,8 @@ class DecoderModel(Part):
     def forward(self, step) -> torch.Tensor:
         """Hidden states after the final norm, for the rows whose logits are wanted only: [n, hidden]."""
         hidden = ops.embed(step.input_ids, self.embed_weight, self.spec.embed_scale)
+        if self.embed_norm is not None:
+            hidden = self.embed_norm.forward(hidden)
         residual = None
         order = self.run_order
         for i, (entry, cache) in enumerate(zip(order, self.cache_views)):

@@ -54,3 +54,26 @@ class RMSNorm(Part):
             return (normed if deferred else normed.tensor()), residual
         y = ops.rmsnorm(x, self.weight, self.eps, residual=residual)
         return y, residual
+
+
+@NORMS.register("scalar_rmsnorm")
+class ScalarRMSNorm(Part):
+    """y = x / sqrt(mean(x^2) + eps) * g with one number g for all coordinates. Statistics and the weight are
+    float32; the rows that come in and go out may differ in element type (``forward(x, out_dtype)``)."""
+
+    def __init__(self, eps: float, output: str = "same"):
+        """``output``: the element type of the result where ``forward`` is not told: "same" as the input,
+        "float32" (a stream carried in float32), or "rows" (the model's element type for rows)."""
+        if output not in ("same", "float32", "rows"):
+            raise ValueError(f"output must be 'same', 'float32' or 'rows', got {output!r}")
+        self.eps, self.output = eps, output
+        self.weight = None
+        self.row_dtype = None         # set when the model's weights are bound
+
+    def param_specs(self):
+        return {"weight": ParamSpec((), init="norm", always_float32=True)}
+
+    def forward(self, x, out_dtype=None) -> torch.Tensor:
+        if out_dtype is None:
+            out_dtype = {"same": x.dtype, "float32": torch.float32, "rows": self.row_dtype or x.dtype}[self.output]
+        return ops.scalar_rmsnorm(x, self.weight, self.eps, out_dtype=out_dtype)

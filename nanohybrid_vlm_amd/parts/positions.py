@@ -66,3 +66,44 @@ class NoPositions(PositionEncoding):
 
     def to(self, device):
         return self
+
+
+@POSITION_ENCODINGS.register("rotary_frequencies")
+class RotaryFrequencies(PositionEncoding):
+    """Rotation given by its frequencies alone: pair i of the first ``rotary_dim`` entries of a head turns by
+    position * f_i, f_i = base^(-2 i / rotary_dim) / scaling_factor (linear scaling: every frequency divided by one
+    number). There is no table: the mixer's kernel takes the angle in float from the position, so no number of
+    positions bounds the model. ``frequencies_for(size)`` gives the unscaled frequencies of the same base over
+    another size (values that are turned over all their entries)."""
+
+    def __init__(self, rotary_dim: int, base: float, max_position: int, scaling_factor: float | None = None, device=None):
+        if rotary_dim % 2 or rotary_dim < 0:
+            raise ValueError(f"rotary_dim must be even and not negative, got {rotary_dim}")
+        if scaling_factor is not None and not scaling_factor > 0:
+            raise ValueError(f"the scaling factor must be positive, got {scaling_factor}")
+        self.rotary_dim, self.base, self.max_position, self.scaling_factor = rotary_dim, float(base), max_position, scaling_factor
+        self.device = device
+        self.freqs = self._frequencies(rotary_dim, scaling_factor)
+        self._others: dict[int, torch.Tensor] = {}
+
+    def _frequencies(self, size: int, factor) -> torch.Tensor:
+        f = self.base ** (-2.0 * torch.arange(size // 2, dtype=torch.float64) / size)
+        if factor is not None:
+            f = f / factor
+        f = f.to(torch.float32)
+        return f.to(self.device) if self.device is not None else f
+
+    def frequencies(self) -> torch.Tensor:
+        """[rotary_dim / 2] float32."""
+        return self.freqs
+
+    def frequencies_for(self, size: int) -> torch.Tensor:
+        if size not in self._others:
+            self._others[size] = self._frequencies(size, None)
+        return self._others[size]
+
+    def to(self, device):
+        self.device = device
+        self.freqs = self.freqs.to(device)
+        self._others = {n: f.to(device) for n, f in self._others.items()}
+        return self

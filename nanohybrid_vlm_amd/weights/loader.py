@@ -10,6 +10,7 @@ tensors it needs and did not get, and tensors of the wrong shape
 
 Element types: a 16-bit tensor becomes bfloat16 (float32 in a float32 run);
 a tensor stored in 32-bit stays float32 if the parameter allows it (norm weights),
+a parameter that enters 32-bit arithmetic only is float32 whatever the file stores,
 integer tables become int32.
 """
 from __future__ import annotations
@@ -51,6 +52,16 @@ def _files(folder: str) -> list[str]:
     if not files:
         raise FileNotFoundError(f"no *.safetensors file in model folder '{folder}'")
     return files
+
+
+def checkpoint_shapes(folder: str) -> dict[str, tuple[int, ...]]:
+    """Name -> shape of every stored tensor; only the files' headers are read."""
+    shapes = {}
+    for path in _files(folder):
+        with safe_open(path, framework="pt", device="cpu") as f:
+            for key in f.keys():
+                shapes[key] = tuple(f.get_slice(key).get_shape())
+    return shapes
 
 
 def load_weights(model, arch, cfg, folder: str, dtype: torch.dtype, device) -> dict[str, torch.Tensor]:
@@ -111,6 +122,8 @@ def load_weights(model, arch, cfg, folder: str, dtype: torch.dtype, device) -> d
         stored = {found[n][1] for n in by_param.get(pname, [])}
         if stored and stored <= _ST_DTYPES_INT:
             pdtype = torch.int32
+        elif spec.always_float32:
+            pdtype = torch.float32
         elif spec.keeps_float32 and stored and stored <= _ST_DTYPES_32:
             pdtype = torch.float32
         else:

@@ -19,7 +19,9 @@ from ..config.registry import resolve_architecture
 _STORE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
 
-def _draw(init: str, shape, gen: torch.Generator) -> torch.Tensor:
+def _draw(init: str, shape, gen: torch.Generator, mean=None, std=None) -> torch.Tensor:
+    if mean is not None or std is not None:
+        return (mean or 0.0) + (0.02 if std is None else std) * torch.randn(shape, generator=gen, dtype=torch.float32)
     if init == "norm":
         return 1.0 + 0.1 * torch.randn(shape, generator=gen, dtype=torch.float32)
     if init in ("normal", "zeros"):
@@ -44,7 +46,7 @@ def random_checkpoint_tensors(raw_config: dict, seed: int, store_dtype: str = "b
         shape = ((src.rows,) + tuple(spec.shape[1:])) if src.rows is not None else tuple(spec.shape)
         gen = torch.Generator(device="cpu")
         gen.manual_seed((int(seed) * 1000003 + index) & 0x7FFFFFFFFFFFFFFF)
-        out[name] = _draw(spec.init, shape, gen).to(_STORE[store_dtype])
+        out[name] = _draw(spec.init, shape, gen, spec.init_mean, spec.init_std).to(_STORE[store_dtype])
     return out
 
 
@@ -78,8 +80,10 @@ def fill_from_device_generator(model, seed: int, dtype: torch.dtype, device) -> 
     params = {}
     for name, spec in model.all_param_specs().items():
         # what a checkpoint would store in 32-bit (norm weights, routers) stays float32 here too
-        t = torch.empty(spec.shape, dtype=torch.float32 if spec.keeps_float32 else dtype, device=device)
-        if spec.init == "norm":
+        t = torch.empty(spec.shape, dtype=torch.float32 if spec.keeps_float32 or spec.always_float32 else dtype, device=device)
+        if spec.init_mean is not None or spec.init_std is not None:
+            t.normal_(spec.init_mean or 0.0, 0.02 if spec.init_std is None else spec.init_std, generator=gen)
+        elif spec.init == "norm":
             t.normal_(1.0, 0.1, generator=gen)
         else:
             t.normal_(0.0, 0.02, generator=gen)

@@ -78,16 +78,18 @@ class EmulatedBackend:
             k_cache.view(-1, Hkv, D)[slots] = k[ok]
             v_cache.view(-1, Hkv, D)[slots] = v[ok].to(dt)
 
-    def paged_attention(self, q, k_cache, v_cache, out, batch, block_tables, scale, window):
+    def paged_attention(self, q, k_cache, v_cache, out, batch, block_tables, scale, window, chunk=0):
         T, Hq, D = q.shape
         page_size, Hkv = k_cache.shape[1], k_cache.shape[2]
         group = Hq // Hkv
-        kf = k_cache.view(-1, Hkv, D)
-        vf = v_cache.view(-1, Hkv, D)
+        kf = k_cache.reshape(-1, Hkv, D)
+        vf = v_cache.reshape(-1, Hkv, v_cache.shape[3])
         for t in range(T):
             r = int(batch.token_req[t])
             p = int(batch.positions[t])
             lo = max(0, p - window + 1) if window > 0 else 0
+            if chunk > 0:
+                lo = p - p % chunk
             kp = torch.arange(lo, p + 1)
             slots = block_tables[r, kp // page_size].long() * page_size + kp % page_size
             for h in range(Hq):
@@ -95,6 +97,124 @@ class EmulatedBackend:
                 vh = vf[slots, h // group].float()
                 s = (kh @ q[t, h].float()) * scale
                 out[t, h] = (torch.softmax(s, dim=0) @ vh).to(out.dtype)
+
+    # -- layers that are not the pre-norm kind
+    def scalar_rmsnorm(self, x, gain, y, eps):
+        s = x.float()
+        y.copy_((s * (gain.float() / torch.sqrt(s.pow(2).mean(-1, keepdim=True) + eps))).to(y.dtype))
+
+    def pair_norm_mean(self, a, wa, b, wb, y, eps):
+        def norm(t, w):
+            t = t.float()
+            return t / torch.sqrt(t.pow(2).mean(-1, keepdim=True) + eps) * w
+        y.copy_((0.5 * (norm(a, wa) + norm(b, wb))).to(y.dtype))
+
+    def depth_mix(self, x, a, b, results, index, weights, out, gain, normed, eps):
+        add = a.float() if b is None else a.float() + b.float()
+        if index == 0:
+            results[0] = x
+        results[index + 1] = x + add
+        total = torch.zeros_like(x)
+        for j in range(index + 2):
+            total = total + weights[j] * results[j]
+        out.copy_(total)
+        if gain is not None:
+            normed.copy_((total * (gain / torch.sqrt(total.pow(2).mean(-1, keepdim=True) + eps))).to(normed.dtype))
+
+    @staticmethod
+    def _turned(t, positions, freqs, sign=1.0):
+        half = freqs.shape[0]
+        ang = sign * positions.float()[:, None] * freqs[None, :]
+        cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        u, v = t[..., :half], t[..., half:2 * half]
+        return torch.cat((u * cos - v * sin, v * cos + u * sin, t[..., 2 * half:]), dim=-1)
+
+    def rotary_split_write(self, qkv, bias, qk_freqs, rot, v_freqs, positions, slot_mapping, q_out, k_cache, v_cache,
+                           Hq, Hkv, D, E, with_kv):
+        T, dt = qkv.shape[0], qkv.dtype
+        x = qkv.float()
+        if bias is not None:
+            x = (x + bias.float()).to(dt).float()
+        q = x[:, :Hq * D].reshape(T, Hq, D)
+        q_out.copy_((self._turned(q, positions, qk_freqs) if rot else q).to(dt))
+        if with_kv:
+            k = x[:, Hq * D:(Hq + Hkv) * D].reshape(T, Hkv, D)
+            v = x[:, (Hq + Hkv) * D:].reshape(T, Hkv, E)
+            if rot:
+                k = self._turned(k, positions, qk_freqs)
+            if v_freqs is not None:
+                v = self._turned(v, positions, v_freqs)
+            ok = slot_mapping >= 0
+            slots = slot_mapping[ok].long()
+            k_cache.view(-1, Hkv, D)[slots] = k[ok].to(dt)
+            v_cache.view(-1, Hkv, E)[slots] = v[ok].to(dt)
+
+    def turn_back(self, x, freqs, positions):
+        x.copy_(self._turned(x.float(), positions, freqs, sign=-1.0).to(x.dtype))
+
+    # -- the gated delta rule: the four kernels, request by request and token by token
+    def delta_prepare(self, proj, taps, kept, a_lin, dt_bias, a_log, batch, state_slots, q, k, v, beta, H, G, D, E):
+        n = taps.shape[1]
+        C = 2 * G * D + H * E
+        x = proj.float()
+        for t in range(proj.shape[0]):
+            r = int(batch.token_req[t])
+            first, pos = int(batch.cu_seqlens_q[r]), int(batch.positions[t])
+            mine = kept[int(state_slots[r])]
+            total = torch.zeros(C)
+            for j in range(n):
+                if pos - j < 0:
+                    break
+                inp = x[t - j, :C] if j <= t - first else mine[:, (n - 1) + (t - first) - j]
+                total = total + taps[:, n - 1 - j] * inp
+            act = total * torch.sigmoid(total)
+            qk = act[:2 * G * D].view(2 * G, D)
+            qk = qk / torch.sqrt(qk.pow(2).sum(-1, keepdim=True) + 1e-6)
+            q[t] = qk[:G] * D ** -0.5
+            k[t] = qk[G:]
+            v[t] = act[2 * G * D:].view(H, E)
+            step = torch.nn.functional.softplus(a_lin[t] + dt_bias, threshold=20.0)
+            a_lin[t] = torch.exp(-torch.exp(a_log).repeat_interleave(D) * step)
+            beta[t] = torch.sigmoid(x[t, C:])
+
+    def conv_state_update(self, proj, kept, n_taps, batch, state_slots, channels):
+        x = proj.float()
+        for r in range(batch.num_requests):
+            first, end = int(batch.cu_seqlens_q[r]), int(batch.cu_seqlens_q[r + 1])
+            n = end - first
+            if n <= 0 or n_taps == 1:
+                continue
+            start = int(batch.positions[first])
+            mine = kept[int(state_slots[r])]
+            old = mine.clone()
+            for s in range(n_taps - 1):
+                rel = n - (n_taps - 1) + s
+                if rel >= 0:
+                    mine[:, s] = x[first + rel, :channels]
+                else:
+                    mine[:, s] = old[:, n + s] if start + rel >= 0 else 0.0
+
+    def delta_rule(self, q, k, v, decay, beta, state, out, batch, state_slots):
+        T, G, D = q.shape
+        H = v.shape[1]
+        for r in range(batch.num_requests):
+            first, end = int(batch.cu_seqlens_q[r]), int(batch.cu_seqlens_q[r + 1])
+            if end <= first:
+                continue
+            slot = int(state_slots[r])
+            for h in range(H):
+                g = h // (H // G)
+                S = torch.zeros_like(state[slot, h]) if int(batch.positions[first]) == 0 else state[slot, h].clone()   # [E, D]
+                for t in range(first, end):
+                    S = S * decay[t, h][None, :]
+                    u = beta[t, h] * (v[t, h] - S @ k[t, g])
+                    S = S + u[:, None] * k[t, g][None, :]
+                    out[t, h] = S @ q[t, g]
+                state[slot, h] = S
+
+    def gated_head_norm(self, o, gate, w, y, eps):
+        r = torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+        y.copy_((o * r * w * torch.sigmoid(gate)).to(y.dtype))
 
     def linear(self, x, w, bias, out):
         y = x.float() @ w.float().T
