@@ -18,6 +18,11 @@ For these two ``value`` is generated tokens a second over the whole run, prompts
 
 ``--workload projections`` is a diagnosis, not the benchmark: a layer's matrix products alone, cold, beside a kernel
 that only reads the same bytes (see ``bench_projections``).
+
+``--workload design --shape pevazen-1b|pevazen-8b [--layers L]``: a model of the Pevazen design (attention and
+recurrent layers side by side, see ``architectures/pevazen.py``) beside a Qwen3 model of the same width, heads,
+feed-forward size, vocabulary and number of layers: one prompt of ``--prompt-tokens`` in one step, decoding at
+``--batch`` requests, and the time of every own kernel in one eager step of each kind (see ``bench_design``).
 """
 import argparse
 import json
@@ -39,7 +44,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=_int_or_list, default=None, help="requests decoding side by side (8b: 8, 14b: 32, 32b: 16)")
     ap.add_argument("--shape", default="8b")
-    ap.add_argument("--workload", default="auto", choices=("auto", "points", "serving", "projections"),
+    ap.add_argument("--workload", default="auto", choices=("auto", "points", "serving", "projections", "design"),
                     help="points: decode at a fixed batch after equal prompts (8b by default); serving: the 14b / 32b workloads; "
                          "projections: a layer's matrix products alone against a kernel that only reads the same bytes")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (same layer sizes)")
@@ -406,6 +411,85 @@ def bench_projections(args):
     return 0
 
 
+def bench_design(args):
+    """A Pevazen model beside a Qwen3 model of equal sizes: prefill of one prompt, decoding at a fixed batch, and the
+    device time of every own kernel in one eager step of each kind (library products are what is left of the step)."""
+    import types
+    import torch
+    from nanohybrid_vlm_amd import LLM, SamplingParams
+    from nanohybrid_vlm_amd.architectures.qwen3 import _shape as qwen3_shape
+    from nanohybrid_vlm_amd.config.registry import named_shapes
+    from nanohybrid_vlm_amd.engine.runner import StepEntry
+    from nanohybrid_vlm_amd.native import ops
+
+    name = args.shape if args.shape.startswith("pevazen") else "pevazen-1b"
+    new = json.loads(json.dumps(named_shapes()[name]))
+    layers = args.layers or min(8, len(new["layers"]))
+    new["layers"] = new["layers"][:layers]
+    a = new["layers"][1]["mixer"]
+    twin = qwen3_shape(layers, new["width"], a["heads"], a["kv_heads"], a["dim"], new["layers"][0]["mlp"]["ff"], vocab=new["vocab"])
+    batch, T = args.batch or 8, args.prompt_tokens or 2048
+    context = args.context or (T + 512)
+    pages = (batch + 1) * -(-context // args.block_size) + 1
+    out = {}
+    for label, raw in (("pevazen", new), ("qwen3", twin)):
+        llm = LLM(raw, random_weights=0, dtype=args.dtype, kvcache_block_size=args.block_size, max_num_seqs=max(batch, 1),
+                  enforce_eager=args.eager, num_kvcache_blocks=pages, max_num_batched_tokens=max(args.token_budget, T, batch),
+                  max_model_len=context, scheduler_policy="prefill_first")
+        cfg = types.SimpleNamespace(vocab_size=llm.runner.vocab_size)
+        pre_s = run_prefill(llm, cfg, T)
+        seconds, _, step_ms = run_decode(llm, cfg, batch, T, args.steps, args.warmup, 1)
+        stats = llm.get_memory_stats()
+        result = {"prefill_ms": round(pre_s * 1e3, 3), "prefill_tok_s": round(T / pre_s, 1),
+                  "decode_ms_per_step": round(seconds / args.steps * 1e3, 4), "decode_tok_s": round(batch * args.steps / seconds, 1),
+                  "weight_bytes": stats["weight_bytes"], "state_pool_bytes": stats["state_pool_bytes"]}
+        # one eager step of each kind with an event around every own kernel
+        runner = llm.runner
+        prompt = random_prompts(1, T, cfg.vocab_size, 77)[0]
+        for kind in ("prefill", "decode"):
+            if kind == "prefill":
+                entries = [StepEntry(("k", 0), prompt, [T - 1])]
+            else:
+                for i in range(batch):
+                    runner.step([StepEntry(("k", 1 + i), prompt, [])])
+                entries = [StepEntry(("k", 1 + i), [1], [0]) for i in range(batch)]
+            graphs, runner.use_graphs = runner.use_graphs, False
+            runner.step(entries)                          # (untimed: libraries loaded, products chosen)
+            for e in entries:
+                runner.finish(e.request_id)
+            if kind == "decode":
+                for i in range(batch):
+                    runner.step([StepEntry(("k", 1 + i), prompt, [])])
+            torch.cuda.synchronize()
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            with ops.kernel_times() as times:
+                start.record()
+                runner.step(entries)
+                end.record()
+            torch.cuda.synchronize()
+            result[f"{kind}_eager_step_ms"] = round(start.elapsed_time(end), 3)
+            result[f"{kind}_kernels_us"] = {k: [n, round(ms / n * 1e3, 1)] for k, (n, ms) in
+                                             sorted(times.summary().items(), key=lambda kv: -kv[1][1])}
+            for e in entries:
+                runner.finish(e.request_id)
+            runner.use_graphs = graphs
+        out[label] = result
+        print(f"{label}: prefill of {T} tokens {result['prefill_ms']} ms, decode at {batch} requests {result['decode_ms_per_step']} ms a step",
+              file=sys.stderr, flush=True)
+        llm.exit()
+        del llm, runner
+        torch.cuda.empty_cache()
+    line = {"metric": f"Pevazen ({name}, {layers} layers) beside Qwen3 of equal sizes: prefill of {T} tokens and decode at batch {batch}",
+            "value": out["pevazen"]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": out["pevazen"]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random token ids, random weights",
+            "config": {"model": name, "layers": layers, "width": new["width"], "global_batch": batch, "prompt_len": T,
+                       "seq_len": context, "parallelism": "single GPU", "graphs": not args.eager},
+            "pevazen": out["pevazen"], "qwen3": out["qwen3"]}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -414,6 +498,8 @@ def main():
     serving = args.workload == "serving" or (args.workload == "auto" and args.shape in ("14b", "32b"))
     if args.workload == "projections":
         return bench_projections(args)
+    if args.workload == "design":
+        return bench_design(args)
     if isinstance(args.batch, str):
         print(f"bench.py: --batch {args.batch}: a list of row counts goes with --workload projections only", flush=True)
         return 2

@@ -74,7 +74,7 @@ __global__ __launch_bounds__(64) void decode_attention_kernel(
   const int kvh = (int)((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x);
   const int G = Hq / Hkv;
   const int pos = positions[t];
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = nhv_first_key(pos, window);
   const int first = max(lo, split * split_len);
   const int last = min(pos, (split + 1) * split_len - 1);
   if (first > last) return;              // this split holds no visible key; the merge knows from pos and lo
@@ -249,7 +249,7 @@ __global__ __launch_bounds__(64 * W) void merge_splits_kernel(const float* __res
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int t = item / Hq;
   const int pos = positions[t];
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = nhv_first_key(pos, window);
   // (the launch's splits must cover every position; one that they do not cover loses its last keys here rather
   // than reading past the splits' results)
   const int s0 = lo / split_len, s1 = min(pos / split_len, n_splits - 1);
@@ -345,7 +345,7 @@ __global__ __launch_bounds__(64 * W) void merge_splits_at_once_kernel(const floa
       v[i][p] = (in && qd < MQ) ? *reinterpret_cast<const float4*>(po + (size_t)s * D + qd * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
   }
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = nhv_first_key(pos, window);
   const int s0 = lo / split_len, s1 = min(pos / split_len, n_splits - 1);
   float m = -INFINITY;
 #pragma unroll
@@ -468,7 +468,6 @@ static int check_decode_attention(int max_blocks, int T, int Hq, int Hkv, int pa
   NHV_REQUIRE(G <= 16, "decode attention: %d query heads per key head are beyond this kernel's limit of 16", G);
   NHV_REQUIRE(split_len > 0 && split_len % RK == 0, "decode attention: split length %d must be a multiple of %d", split_len, RK);
   NHV_REQUIRE(n_splits > 0 && n_splits <= 65535 && Hkv <= 65535 && T <= 65535, "decode attention: grid too large");
-  NHV_REQUIRE(window >= 0, "decode attention: negative window");
   return 0;
 }
 

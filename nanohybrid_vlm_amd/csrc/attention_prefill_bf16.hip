@@ -30,7 +30,8 @@
 // element i % 4 of the 8-byte pieces that lanes i / 4 + 4 j (j = 0..3) point at, so with
 // lane r pointing at key r / 4, entries 4 (r % 4).. of the 16-entry block, lane i gets
 // entry i of four consecutive keys. A query at position p reads keys lo..p (lo = p -
-// window + 1 with a window, else 0). Keys outside the block's range are replaced by the
+// window + 1 with a window, the start of p's own block of positions with a chunk, which
+// comes as a negative window, else 0). Keys outside the block's range are replaced by the
 // nearest key inside it (their P is 0): unused cache slots may hold anything, and 0 * NaN
 // would poison the sums.
 #include "nhv_common.h"
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
   const int blk_tok_lo = (first_tile / G) * 16;
   const int blk_tok_hi = min((last_tile / G) * 16 + 15, q_len - 1);
   const int key_hi = start_pos + blk_tok_hi;
-  const int key_lo = window > 0 ? max(0, start_pos + blk_tok_lo - window + 1) : 0;
+  const int key_lo = nhv_first_key(start_pos + blk_tok_lo, window);
 
   // this wave's row tiles; this lane's row (in both products) is token tok0 + col of the tile's head
   const bool live = first_tile + wave * RT < n_row_tiles;
@@ -151,12 +152,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     row_tok[r] = tok0 + col;
     row_ok[r] = tile_live && row_tok[r] < q_len;
     row_pos[r] = tile_live ? start_pos + min(row_tok[r], q_len - 1) : -1;    // a tile beyond the portion sees no key
-    row_lo[r] = window > 0 ? max(0, row_pos[r] - window + 1) : 0;
+    row_lo[r] = nhv_first_key(row_pos[r], window);
     if (tile_live) {
       const int hi = start_pos + min(tok0 + 15, q_len - 1);                 // beyond it the tile has nothing to do
       wave_lo_pos = min(wave_lo_pos, start_pos + tok0);                       // the tile's first row sees the fewest keys
       wave_hi = max(wave_hi, hi);
-      wave_max_lo = max(wave_max_lo, window > 0 ? max(0, hi - window + 1) : 0);
+      wave_max_lo = max(wave_max_lo, nhv_first_key(hi, window));
     }
 #pragma unroll
     for (int s = 0; s < DSTEPS; ++s) {
@@ -387,7 +388,6 @@ extern "C" int nhv_prefill_attention_bf16(const void* q, const void* k_cache, co
                                           int window, void* stream) {
   NHV_REQUIRE(B > 0 && max_q_len > 0 && Hq > 0 && Hkv > 0 && page_size > 0 && max_blocks > 0, "prefill attention: bad sizes");
   NHV_REQUIRE(Hq % Hkv == 0, "prefill attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
-  NHV_REQUIRE(window >= 0, "prefill attention: negative window");
   NHV_REQUIRE(prefill::SUPPORTED, "prefill attention: head size %d is beyond this kernel's limit of 256", prefill::D);
   int page_shift = -1;
   for (int b = 0; b < 31; ++b)

@@ -10,8 +10,8 @@
 //  - nhv_gated_head_norm: per (token, head), o over its root mean square, times a weight, times sigmoid(gate).
 // Everything here is float: the state, the decays, the unit vectors, the sums. A column of S (one value channel)
 // never meets another column, so a block owns a tile of columns, a column belongs to R adjacent lanes that hold D / R
-// entries each, and the two sums over D per token are taken with lane shuffles; the next token's vectors are asked
-// for before this token's are used. A request without tokens in the step is left alone.
+// entries each, and the two sums over D per token are taken with lane shuffles; the tokens' vectors come through
+// LDS a tile of tokens ahead. A request without tokens in the step is left alone.
 #include "nhv_common.h"
 #include <math.h>
 
@@ -25,6 +25,8 @@ __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log
 // proj[T, ld]: q (G D) | k (G D) | v (H E) | beta (H) as the projection left them. taps[C, n], C = 2 G D + H E, last
 // column for the token itself. kept[slots, C, n - 1]: the inputs at the n - 1 positions before the request's first
 // token of this step. a_lin[T, H D]: the decays' linear part on entry, the decays on return.
+// One wave per (token, unit); the units of a token are its 2 G query and key heads (D channels each), its H value
+// heads (E channels), its H heads of decays (D channels) and its H betas (one unit).
 template <typename TI>
 __global__ __launch_bounds__(256) void delta_prepare_kernel(
     const TI* __restrict__ proj, int ld, const float* __restrict__ taps, int n_taps, const float* __restrict__ kept,
@@ -32,45 +34,63 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
     const int* __restrict__ token_req, const int* __restrict__ positions, const int* __restrict__ cu,
     const int* __restrict__ state_slots, float* __restrict__ q_out, float* __restrict__ k_out, float* __restrict__ v_out,
     float* __restrict__ beta_out, int H, int G, int D, int E) {
-  extern __shared__ float conv[];            // C floats
-  const int t = blockIdx.x;
-  const int req = token_req[t];
-  const int first = cu[req];
-  const int i_in_step = t - first;           // tokens of this request before this one in the step
-  const int pos = positions[t];
+  const int t = blockIdx.y;
+  const int lane = threadIdx.x & 63;
+  const int unit = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int n_units = 2 * G + 2 * H + 1;
+  if (unit >= n_units) return;
   const int C = 2 * G * D + H * E;
-  const float* mine = kept + (size_t)state_slots[req] * C * (n_taps - 1);
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float sum = 0.f;
-    for (int j = 0; j < n_taps; ++j) {       // the input j positions back meets the tap n - 1 - j
-      if (pos - j < 0) break;
-      float x;
-      if (j <= i_in_step) x = to_f32(proj[(size_t)(t - j) * ld + c]);
-      else x = mine[(size_t)c * (n_taps - 1) + (n_taps - 1) + i_in_step - j];
-      sum = fmaf(taps[(size_t)c * n_taps + n_taps - 1 - j], x, sum);
+  if (unit == n_units - 1) {
+    for (int h = lane; h < H; h += NHV_WAVE) beta_out[(size_t)t * H + h] = sigmoid_f(to_f32(proj[(size_t)t * ld + C + h]));
+    return;
+  }
+  if (unit >= 2 * G + H) {
+    const int h = unit - 2 * G - H;
+    const float rate = expf(a_log[h]);
+    for (int d = lane; d < D; d += NHV_WAVE) {
+      const size_t at = (size_t)t * H * D + h * D + d;
+      a_lin[at] = expf(-rate * softplus_f(a_lin[at] + dt_bias[h * D + d]));
     }
-    conv[c] = silu_f(sum);
+    return;
   }
-  __syncthreads();
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
-  // q and k heads: unit length (the sum of squares plus 1e-6 under the root); q also times D^(-1/2)
-  const float q_scale = 1.0f / sqrtf((float)D);
-  for (int head = wave; head < 2 * G; head += n_waves) {
-    const float* src = conv + head * D;
-    float ss = 0.f;
-    for (int d = lane; d < D; d += NHV_WAVE) ss = fmaf(src[d], src[d], ss);
-    ss = wave_sum(ss);
-    const float r = (head < G ? q_scale : 1.0f) / sqrtf(ss + 1e-6f);
-    float* dst = head < G ? q_out + ((size_t)t * G + head) * D : k_out + ((size_t)t * G + head - G) * D;
-    for (int d = lane; d < D; d += NHV_WAVE) dst[d] = src[d] * r;
+  const int req = token_req[t];
+  const int i_in_step = t - cu[req];         // tokens of this request before this one in the step
+  const int pos = positions[t];
+  const float* mine = kept + (size_t)state_slots[req] * C * (n_taps - 1);
+  const bool is_v = unit >= 2 * G;
+  const int size = is_v ? E : D;
+  const int c0 = is_v ? 2 * G * D + (unit - 2 * G) * E : unit * D;
+  float vals[16];                            // (heads of up to 1024 channels)
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int d = lane + i * NHV_WAVE;
+    vals[i] = 0.f;
+    if (d < size) {
+      const int c = c0 + d;
+      float sum = 0.f;
+      for (int j = 0; j < n_taps; ++j) {     // the input j positions back meets the tap n - 1 - j
+        if (pos - j < 0) break;
+        const float x = j <= i_in_step ? to_f32(proj[(size_t)(t - j) * ld + c])
+                                       : mine[(size_t)c * (n_taps - 1) + (n_taps - 1) + i_in_step - j];
+        sum = fmaf(taps[(size_t)c * n_taps + n_taps - 1 - j], x, sum);
+      }
+      vals[i] = silu_f(sum);
+      ss = fmaf(vals[i], vals[i], ss);
+    }
   }
-  for (int c = threadIdx.x; c < H * E; c += blockDim.x) v_out[(size_t)t * H * E + c] = conv[2 * G * D + c];
-  for (int c = threadIdx.x; c < H * D; c += blockDim.x) {
-    const float step = softplus_f(a_lin[(size_t)t * H * D + c] + dt_bias[c]);
-    a_lin[(size_t)t * H * D + c] = expf(-expf(a_log[c / D]) * step);
+  float r = 1.0f;
+  float* dst = v_out + (size_t)t * H * E + (c0 - 2 * G * D);
+  if (!is_v) {
+    // unit length (the sum of squares plus 1e-6 under the root); q also times D^(-1/2)
+    r = (unit < G ? 1.0f / sqrtf((float)D) : 1.0f) / sqrtf(wave_sum(ss) + 1e-6f);
+    dst = unit < G ? q_out + ((size_t)t * G + unit) * D : k_out + ((size_t)t * G + unit - G) * D;
   }
-  for (int h = threadIdx.x; h < H; h += blockDim.x)
-    beta_out[(size_t)t * H + h] = sigmoid_f(to_f32(proj[(size_t)t * ld + C + h]));
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int d = lane + i * NHV_WAVE;
+    if (d < size) dst[d] = vals[i] * r;
+  }
 }
 
 extern "C" int nhv_delta_prepare(const void* proj, int proj_dtype, const void* taps, int n_taps, const void* kept,
@@ -79,19 +99,15 @@ extern "C" int nhv_delta_prepare(const void* proj, int proj_dtype, const void* t
                                  void* v_out, void* beta_out, int T, int H, int G, int D, int E, void* stream) {
   NHV_REQUIRE(T > 0 && H > 0 && G > 0 && D > 0 && E > 0 && H % G == 0, "delta_prepare: bad sizes T=%d H=%d G=%d D=%d E=%d", T, H, G, D, E);
   NHV_REQUIRE(n_taps >= 1 && n_taps <= NHV_MAX_TAPS, "delta_prepare: %d taps (1 to %d are taken)", n_taps, NHV_MAX_TAPS);
+  NHV_REQUIRE(D <= 1024 && E <= 1024 && T <= 65535, "delta_prepare: D=%d, E=%d (up to 1024 each), T=%d (up to 65535 a call)", D, E, T);
   const int C = 2 * G * D + H * E;
-  const size_t lds = (size_t)C * sizeof(float);
-  NHV_REQUIRE(lds <= 160 * 1024, "delta_prepare: %d channels do not fit a block's scratch memory", C);
+  const int n_units = 2 * G + 2 * H + 1;
   hipStream_t s = (hipStream_t)stream;
 #define LAUNCH(TI)                                                                                                    \
-  do {                                                                                                                \
-    if (lds > 64 * 1024)                                                                                              \
-      (void)hipFuncSetAttribute((const void*)delta_prepare_kernel<TI>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
-    hipLaunchKernelGGL(delta_prepare_kernel<TI>, dim3(T), dim3(256), lds, s, (const TI*)proj, C + H, (const float*)taps, \
-                       n_taps, (const float*)kept, (float*)a_lin, (const float*)dt_bias, (const float*)a_log,         \
-                       (const int*)token_req, (const int*)positions, (const int*)cu, (const int*)state_slots,         \
-                       (float*)q_out, (float*)k_out, (float*)v_out, (float*)beta_out, H, G, D, E);                    \
-  } while (0)
+  hipLaunchKernelGGL(delta_prepare_kernel<TI>, dim3((n_units + 3) / 4, T), dim3(256), 0, s, (const TI*)proj, C + H,   \
+                     (const float*)taps, n_taps, (const float*)kept, (float*)a_lin, (const float*)dt_bias,            \
+                     (const float*)a_log, (const int*)token_req, (const int*)positions, (const int*)cu,               \
+                     (const int*)state_slots, (float*)q_out, (float*)k_out, (float*)v_out, (float*)beta_out, H, G, D, E)
   if (proj_dtype == NHV_F32) LAUNCH(float);
   else if (proj_dtype == NHV_BF16) LAUNCH(bf16_t);
   else return nhv_fail("delta_prepare: unknown dtype %d", proj_dtype);
@@ -144,64 +160,138 @@ extern "C" int nhv_conv_state_update(const void* proj, int proj_dtype, int ld, v
 // ---------------------------------------------------------------- the recurrence
 // state[slots, H, E, D]: a column of S lies contiguous. Thread (column e, part r) of a block holds S[r DR .. r DR + DR, e];
 // the R parts of a column are adjacent lanes (R a power of two, at most 64). Entries beyond D (where D is no multiple
-// of R DR) are zeros that change nothing.
+// of R DR) are zeros that change nothing. The tokens' vectors (q, k, the decays: D floats each; the block's columns of
+// v; beta) come through LDS in tiles of ``tile`` tokens, two buffers: the next tile's loads are under way in registers
+// while this tile is computed, and are stored when it is done; one barrier a tile. A token then costs its
+// arithmetic and two sums over R lanes, not a trip to memory.
+#define NHV_DELTA_STAGE 12     // floats a thread can hold of the next tile (a tile has at most 256 * this many)
+
+// The sum of x over the R adjacent lanes of a column (R a power of two, the groups aligned), in every one of them.
+// Within a row of 16 lanes the partners are reached by lane permutations inside the instruction itself (the two
+// exchanges inside a group of four; then, all four being equal, the mirror images within eight and within sixteen
+// lanes); only beyond sixteen lanes do values cross through the permute unit.
+__device__ __forceinline__ float column_sum(float x, int R) {
+#define NHV_DPP_ADD(ctrl) x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), ctrl, 0xf, 0xf, true))
+  if (R > 1) NHV_DPP_ADD(0xB1);        // quad_perm [1, 0, 3, 2]
+  if (R > 2) NHV_DPP_ADD(0x4E);        // quad_perm [2, 3, 0, 1]
+  if (R > 4) NHV_DPP_ADD(0x141);       // row_half_mirror
+  if (R > 8) NHV_DPP_ADD(0x140);       // row_mirror
+#undef NHV_DPP_ADD
+  if (R > 16) x += __shfl_xor(x, 16, NHV_WAVE);
+  if (R > 32) x += __shfl_xor(x, 32, NHV_WAVE);
+  return x;
+}
+
 template <int DR>
 __global__ __launch_bounds__(256) void delta_rule_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, const float* __restrict__ decay,
     const float* __restrict__ beta, float* __restrict__ state, float* __restrict__ out, const int* __restrict__ positions,
-    const int* __restrict__ cu, const int* __restrict__ state_slots, int H, int G, int D, int E, int R, int cols) {
+    const int* __restrict__ cu, const int* __restrict__ state_slots, int H, int G, int D, int E, int R, int cols, int tile) {
+  extern __shared__ __attribute__((aligned(16))) float staged[];   // 2 buffers of tile * row floats, row = 3 Dp + cols + 1 (rounded up to 4), Dp = R DR
   const int req = blockIdx.z, h = blockIdx.y;
   const int first = cu[req], end = cu[req + 1];
   if (end <= first) return;                  // (the same for the whole block)
-  const int e = blockIdx.x * cols + threadIdx.x / R;
+  const int e0 = blockIdx.x * cols;
+  const int e = e0 + threadIdx.x / R;
   const int r = threadIdx.x % R;
   const int d0 = r * DR;
   const bool column = e < E;
   const int g = h / (H / G);
+  const int Dp = R * DR;
+  const int row = 3 * Dp + ((cols + 1 + 3) & ~3);       // (a multiple of four floats: every token's vectors can be read four at a time)
+  const int n_threads = blockDim.x;
   float S[DR];
   float* mine = state + (((size_t)state_slots[req] * H + h) * E + (column ? e : 0)) * D;
   const bool fresh = positions[first] == 0;
 #pragma unroll
   for (int i = 0; i < DR; ++i) S[i] = (!fresh && column && d0 + i < D) ? mine[d0 + i] : 0.f;
 
-  float nq[DR], nk[DR], ng[DR], nv, nb;
-  auto fetch = [&](int t) {
-    const float* qr = q + ((size_t)t * G + g) * D;
-    const float* kr = k + ((size_t)t * G + g) * D;
-    const float* gr = decay + ((size_t)t * H + h) * D;
+  // what this thread brings of a tile: entry x of the tile's tile * row floats, x = threadIdx.x + j * n_threads. Which
+  // token of the tile and which number of it that is does not change from tile to tile: worked out once.
+  float hold[NHV_DELTA_STAGE];
+  const float* src[NHV_DELTA_STAGE];         // where entry j of the tile that begins at token 0 lies (null: a zero)
+  int stride[NHV_DELTA_STAGE], tok_of[NHV_DELTA_STAGE];
 #pragma unroll
-    for (int i = 0; i < DR; ++i) {
-      const bool ok = d0 + i < D;
-      nq[i] = ok ? qr[d0 + i] : 0.f;
-      nk[i] = ok ? kr[d0 + i] : 0.f;
-      ng[i] = ok ? gr[d0 + i] : 0.f;
+  for (int j = 0; j < NHV_DELTA_STAGE; ++j) {
+    const int x = threadIdx.x + j * n_threads;
+    const int tt = x / row, c = x % row;
+    tok_of[j] = tt;
+    src[j] = nullptr;
+    stride[j] = 0;
+    if (tt < tile) {
+      if (c < 3 * Dp) {
+        const int which = c / Dp, d = c % Dp;
+        if (d < D) {
+          src[j] = which == 0 ? q + ((size_t)tt * G + g) * D + d : which == 1 ? k + ((size_t)tt * G + g) * D + d
+                                                                              : decay + ((size_t)tt * H + h) * D + d;
+          stride[j] = which == 2 ? H * D : G * D;
+        }
+      } else if (c < 3 * Dp + cols) {
+        const int ee = e0 + c - 3 * Dp;
+        if (ee < E) {
+          src[j] = v + ((size_t)tt * H + h) * E + ee;
+          stride[j] = H * E;
+        }
+      } else {
+        src[j] = beta + (size_t)tt * H + h;
+        stride[j] = H;
+      }
     }
-    nv = column ? v[((size_t)t * H + h) * E + e] : 0.f;
-    nb = beta[(size_t)t * H + h];
+  }
+  auto ask = [&](int t0, int n) {
+#pragma unroll
+    for (int j = 0; j < NHV_DELTA_STAGE; ++j)
+      hold[j] = (src[j] != nullptr && tok_of[j] < n) ? src[j][(size_t)t0 * stride[j]] : 0.f;
   };
-  fetch(first);
-  for (int t = first; t < end; ++t) {
-    float cq[DR], ck[DR];
-    const float cv = nv, cb = nb;
-    float dot = 0.f;
+  auto put = [&](float* buf, int n) {
 #pragma unroll
-    for (int i = 0; i < DR; ++i) {
-      cq[i] = nq[i];
-      ck[i] = nk[i];
-      S[i] *= ng[i];
-      dot = fmaf(ck[i], S[i], dot);
-    }
-    if (t + 1 < end) fetch(t + 1);
-    for (int o = 1; o < R; o <<= 1) dot += __shfl_xor(dot, o, NHV_WAVE);
-    const float u = cb * (cv - dot);
-    float read = 0.f;
+    for (int j = 0; j < NHV_DELTA_STAGE; ++j)
+      if (tok_of[j] < n) buf[threadIdx.x + j * n_threads] = hold[j];
+  };
+  int n_here = min(tile, end - first);
+  ask(first, n_here);
+  put(staged, n_here);
+  __syncthreads();
+  int cur = 0;
+  for (int t0 = first; t0 < end; t0 += tile) {
+    const int n = min(tile, end - t0);
+    const int n_next = min(tile, end - t0 - tile);
+    if (n_next > 0) ask(t0 + tile, n_next);
+    const float* buf = staged + cur * tile * row;
+    for (int i_t = 0; i_t < n; ++i_t) {
+      const float* tok = buf + i_t * row;
+      // with S' = diag(g) S:  u = beta (v - k . S'),  o = q . (S' + k u) = q . S' + (q . k) u: the three sums over D are
+      // taken together, so a token waits for one exchange between the lanes of its column, not two
+      float ck[DR];
+      float k_s = 0.f, q_s = 0.f, q_k = 0.f;
 #pragma unroll
-    for (int i = 0; i < DR; ++i) {
-      S[i] = fmaf(ck[i], u, S[i]);
-      read = fmaf(cq[i], S[i], read);
+      for (int i = 0; i < DR; i += 4) {
+        const float4 q4 = *reinterpret_cast<const float4*>(tok + d0 + i);
+        const float4 k4 = *reinterpret_cast<const float4*>(tok + Dp + d0 + i);
+        const float4 g4 = *reinterpret_cast<const float4*>(tok + 2 * Dp + d0 + i);
+        const float qv[4] = {q4.x, q4.y, q4.z, q4.w}, kv[4] = {k4.x, k4.y, k4.z, k4.w}, gv[4] = {g4.x, g4.y, g4.z, g4.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          ck[i + j] = kv[j];
+          S[i + j] *= gv[j];
+          k_s = fmaf(kv[j], S[i + j], k_s);
+          q_s = fmaf(qv[j], S[i + j], q_s);
+          q_k = fmaf(qv[j], kv[j], q_k);
+        }
+      }
+      const float cv = tok[3 * Dp + threadIdx.x / R], cb = tok[3 * Dp + cols];
+      k_s = column_sum(k_s, R);
+      q_s = column_sum(q_s, R);
+      q_k = column_sum(q_k, R);
+      const float u = cb * (cv - k_s);
+      const float read = fmaf(q_k, u, q_s);
+#pragma unroll
+      for (int i = 0; i < DR; ++i) S[i] = fmaf(ck[i], u, S[i]);
+      if (r == 0 && column) out[((size_t)(t0 + i_t) * H + h) * E + e] = read;
     }
-    for (int o = 1; o < R; o <<= 1) read += __shfl_xor(read, o, NHV_WAVE);
-    if (r == 0 && column) out[((size_t)t * H + h) * E + e] = read;
+    if (n_next > 0) put(staged + (cur ^ 1) * tile * row, n_next);
+    __syncthreads();
+    cur ^= 1;
   }
   if (column) {
 #pragma unroll
@@ -212,7 +302,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
 
 extern "C" int nhv_delta_rule(const void* q, const void* k, const void* v, const void* decay, const void* beta, void* state,
                               void* out, const void* positions, const void* cu, const void* state_slots, int B, int H, int G,
-                              int D, int E, void* stream) {
+                              int D, int E, int max_q_len, void* stream) {
   NHV_REQUIRE(B > 0 && H > 0 && G > 0 && D > 0 && E > 0 && H % G == 0, "delta_rule: bad sizes B=%d H=%d G=%d D=%d E=%d", B, H, G, D, E);
   NHV_REQUIRE(D <= 1024 && B <= 65535 && H <= 65535, "delta_rule: D=%d (up to 1024), B=%d, H=%d (up to 65535)", D, B, H);
   // entries a lane: 8 from a key size of 64 on, 4 below, 16 where 8 would need more than 64 lanes a column
@@ -222,12 +312,21 @@ extern "C" int nhv_delta_rule(const void* q, const void* k, const void* v, const
   int cols = 256 / R;
   if (cols < 1) cols = 1;
   if (cols > E) cols = E;
-  const dim3 grid((E + cols - 1) / cols, H, B), block(cols * R);
+  const int n_threads = cols * R;
+  const int row = 3 * R * dr + ((cols + 1 + 3) & ~3);
+  // tokens a tile: what the threads can hold of the next tile, at most 16, no more than the longest portion
+  int tile = n_threads * NHV_DELTA_STAGE / row;
+  if (tile > 16) tile = 16;
+  if (tile > max_q_len) tile = max_q_len;
+  if (tile < 1) tile = 1;
+  NHV_REQUIRE(row <= n_threads * NHV_DELTA_STAGE, "delta_rule: a token's %d floats do not fit the block's staging", row);
+  const size_t lds = 2 * (size_t)tile * row * sizeof(float);
+  const dim3 grid((E + cols - 1) / cols, H, B), block(n_threads);
   hipStream_t s = (hipStream_t)stream;
 #define LAUNCH(DRV)                                                                                                   \
-  hipLaunchKernelGGL(delta_rule_kernel<DRV>, grid, block, 0, s, (const float*)q, (const float*)k, (const float*)v,    \
+  hipLaunchKernelGGL(delta_rule_kernel<DRV>, grid, block, lds, s, (const float*)q, (const float*)k, (const float*)v,  \
                      (const float*)decay, (const float*)beta, (float*)state, (float*)out, (const int*)positions,      \
-                     (const int*)cu, (const int*)state_slots, H, G, D, E, R, cols)
+                     (const int*)cu, (const int*)state_slots, H, G, D, E, R, cols, tile)
   if (dr == 16) LAUNCH(16);
   else if (dr == 8) LAUNCH(8);
   else LAUNCH(4);

@@ -24,6 +24,14 @@ int nhv_fail(const char* fmt, ...);
     if (e_ != hipSuccess) return nhv_fail("%s: launch failed: %s", name, hipGetErrorString(e_)); \
   } while (0)
 
+// The first key that the query at position ``pos`` reads. reach 0: all keys; reach n > 0: the last n keys (a window);
+// reach -n < 0: the keys of its own block of n positions, blocks counted from position 0 (a chunk).
+__host__ __device__ __forceinline__ int nhv_first_key(int pos, int reach) {
+  if (reach > 0) return pos - reach + 1 > 0 ? pos - reach + 1 : 0;
+  if (reach < 0) return pos >= 0 ? pos - pos % (-reach) : 0;
+  return 0;
+}
+
 template <typename T>
 __device__ __forceinline__ float to_f32(T v) { return (float)v; }
 template <typename T>

@@ -179,8 +179,10 @@ class NativeBackend:
         T, Hq, D = q.shape
         _, page_size, Hkv, _ = k_cache.shape
         E = v_cache.shape[3]
-        # the kernels on the matrix cores take value heads of the key heads' size and a window or no bound at all
-        fast = q.dtype == torch.bfloat16 and E == D and not chunk and D % 16 == 0 and D <= 256
+        # the kernels on the matrix cores take value heads of the key heads' size; a chunk goes to them as a negative window
+        fast = q.dtype == torch.bfloat16 and E == D and D % 16 == 0 and D <= 256
+        if chunk:
+            window = -chunk
         if fast and batch.max_q_len == 1 and Hq // Hkv <= 16 and T <= 65535:
             return self._decode_attention(q, k_cache, v_cache, out, batch, block_tables, scale, window)
         if fast and batch.num_requests <= 65535 and Hkv <= 65535:
@@ -191,7 +193,7 @@ class NativeBackend:
                               ctypes.c_float(scale), window, _stream(), lib=self.attention_lib(D))
         self._call("nhv_paged_attention_generic", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out),
                    _ptr(batch.token_req), _ptr(batch.positions), _ptr(block_tables), block_tables.shape[1], T, Hq, Hkv,
-                   D, E, page_size, ctypes.c_float(scale), window, chunk, dtype_code(q), _stream())
+                   D, E, page_size, ctypes.c_float(scale), 0 if chunk else window, chunk, dtype_code(q), _stream())
 
     # -- layers that are not the pre-norm kind: norms with one number, sums over depth, rotation without a table --
     def scalar_rmsnorm(self, x, gain, y, eps):
@@ -235,7 +237,7 @@ class NativeBackend:
         _, H, E = v.shape
         self._call("nhv_delta_rule", _ptr(q), _ptr(k), _ptr(v), _ptr(decay), _ptr(beta), _ptr(state), _ptr(out),
                    _ptr(batch.positions), _ptr(batch.cu_seqlens_q), _ptr(state_slots), batch.num_requests, H, G, D, E,
-                   _stream())
+                   max(1, batch.max_q_len), _stream())
 
     def gated_head_norm(self, o, gate, w, y, eps):
         T, H, E = o.shape
@@ -248,8 +250,8 @@ class NativeBackend:
         _, page_size, Hkv, _ = k_cache.shape
         # inside a graph the lengths are only bounded (by max_model_len): the recorder says what to plan for
         span = min(self.planned_context, batch.max_context_len) if self.planned_context else batch.max_context_len
-        if window:
-            span = min(span, window + 64)
+        if window:                                   # (a chunk comes as a negative window)
+            span = min(span, abs(window) + 64)
         # One wave per SIMD of the chip (about a thousand) is the fastest while that leaves splits of up to 256
         # keys, half as many waves again from there on (a wave takes its keys one round after the other), and no
         # split is longer than 1,024 keys. Measured at 2,176 and 8,192 keys, 1 to 64 requests, 8 key/value heads: the

@@ -156,14 +156,17 @@ def _plain_attention(m, q_in, k_in, v_in, rotate_values):
 
 @pytest.mark.parametrize("where", WHERE)
 @pytest.mark.parametrize("rotate_values", [False, True])
-def test_chunked_attention_alone(where, kernels, rotate_values):
+@pytest.mark.parametrize("sizes", [(12, 20), (32, 32)], ids=["D12-E20", "D32-E32"])
+def test_chunked_attention_alone(where, kernels, rotate_values, sizes):
     """Random queries, keys and values; a partial rotation with scaled frequencies; value heads of another size than
-    the key heads; portions that end inside pages and inside chunks."""
+    the key heads, and of the same size in steps of 16 (which the kernels on the matrix cores take in bfloat16);
+    portions that end inside pages and inside chunks."""
     device, dtype = where
-    m = pc._attention(6, 2, 12, 20, 7, 8, 300.0, 0.35, factor=2.5)
+    D, E = sizes
+    m = pc._attention(6, 2, D, E, 7, 8, 300.0, 0.35, factor=2.5)
     g = torch.Generator().manual_seed(5)
     T = 45
-    q_in, k_in, v_in = torch.randn(T, 72, generator=g), torch.randn(T, 24, generator=g), torch.randn(T, 40, generator=g)
+    q_in, k_in, v_in = torch.randn(T, 6 * D, generator=g), torch.randn(T, 2 * D, generator=g), torch.randn(T, 2 * E, generator=g)
     if dtype == "bfloat16":
         q_in, k_in, v_in = (t.bfloat16().float() for t in (q_in, k_in, v_in))
     want = _plain_attention(m, q_in, k_in, v_in, rotate_values)
@@ -173,13 +176,15 @@ def test_chunked_attention_alone(where, kernels, rotate_values):
 
 
 @pytest.mark.parametrize("where", WHERE)
-def test_one_key_that_stands_out(where, kernels):
+@pytest.mark.parametrize("E", [6, 16], ids=["values of their own size", "values of the keys' size"])
+def test_one_key_that_stands_out(where, kernels, E):
     """Among 300 keys one is made to carry nearly all the weight of every query that sees it; its value is a
     vector no other key has. A query then returns that value exactly when the key lies in its own chunk at or
     before it: for the marked key at the first and the last place of a chunk, at a page's border, far back, and for
-    queries just inside and just outside, in a prompt and decoded one by one. No rotation, so the scores are known."""
+    queries just inside and just outside, in a prompt and decoded one by one. No rotation, so the scores are known.
+    (With value heads of the key heads' size the bfloat16 run takes the kernels on the matrix cores.)"""
     device, dtype = where
-    chunk, page, T, D, E = 48, 16, 300, 16, 6
+    chunk, page, T, D = 48, 16, 300, 16
     m = pc._attention(2, 1, D, E, chunk, 0, 10.0, 1.0)
     for marked in (0, 47, 48, 95, 96, 143, 144, 191, 240, 287):
         g = torch.Generator().manual_seed(marked)
@@ -188,7 +193,7 @@ def test_one_key_that_stands_out(where, kernels):
         v_in = 0.1 * torch.randn(T, E, generator=g)
         q_in[:, 0] = q_in[:, D] = 4.0                 # every query asks for coordinate 0 ...
         k_in[marked, 0] = 8.0                         # ... which only the marked key has: its score is 32 above the rest
-        v_in[marked] = torch.tensor([5.0, -5.0, 5.0, -5.0, 5.0, -5.0])
+        v_in[marked] = torch.tensor([5.0, -5.0] * (E // 2))
         for portions in ([T], [marked + 1] + [1] * (T - marked - 1) if marked < 200 else [T - 40] + [1] * 40):
             got = _attention_through_kernels(device, dtype, m, q_in, k_in, v_in, portions, page, False)
             sees = torch.tensor([marked <= i and i // chunk == marked // chunk for i in range(T)])
