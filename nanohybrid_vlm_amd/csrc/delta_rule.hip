@@ -170,7 +170,8 @@ extern "C" int nhv_conv_state_update(const void* proj, int proj_dtype, int ld, v
 // Within a row of 16 lanes the partners are reached by lane permutations inside the instruction itself (the two
 // exchanges inside a group of four; then, all four being equal, the mirror images within eight and within sixteen
 // lanes); only beyond sixteen lanes do values cross through the permute unit.
-__device__ __forceinline__ float column_sum(float x, int R) {
+template <int R>
+__device__ __forceinline__ float column_sum(float x) {
 #define NHV_DPP_ADD(ctrl) x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), ctrl, 0xf, 0xf, true))
   if (R > 1) NHV_DPP_ADD(0xB1);        // quad_perm [1, 0, 3, 2]
   if (R > 2) NHV_DPP_ADD(0x4E);        // quad_perm [2, 3, 0, 1]
@@ -182,11 +183,11 @@ __device__ __forceinline__ float column_sum(float x, int R) {
   return x;
 }
 
-template <int DR>
+template <int DR, int R>
 __global__ __launch_bounds__(256) void delta_rule_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, const float* __restrict__ decay,
     const float* __restrict__ beta, float* __restrict__ state, float* __restrict__ out, const int* __restrict__ positions,
-    const int* __restrict__ cu, const int* __restrict__ state_slots, int H, int G, int D, int E, int R, int cols, int tile) {
+    const int* __restrict__ cu, const int* __restrict__ state_slots, int H, int G, int D, int E, int cols, int tile) {
   extern __shared__ __attribute__((aligned(16))) float staged[];   // 2 buffers of tile * row floats, row = 3 Dp + cols + 1 (rounded up to 4), Dp = R DR
   const int req = blockIdx.z, h = blockIdx.y;
   const int first = cu[req], end = cu[req + 1];
@@ -200,6 +201,9 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
   const int Dp = R * DR;
   const int row = 3 * Dp + ((cols + 1 + 3) & ~3);       // (a multiple of four floats: every token's vectors can be read four at a time)
   const int n_threads = blockDim.x;
+  const int my_col = threadIdx.x / R;
+  const bool writes = r == 0 && column;
+  float* out_col = out + (size_t)h * E + (column ? e : 0);
   float S[DR];
   float* mine = state + (((size_t)state_slots[req] * H + h) * E + (column ? e : 0)) * D;
   const bool fresh = positions[first] == 0;
@@ -243,53 +247,64 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
     for (int j = 0; j < NHV_DELTA_STAGE; ++j)
       hold[j] = (src[j] != nullptr && tok_of[j] < n) ? src[j][(size_t)t0 * stride[j]] : 0.f;
   };
-  auto put = [&](float* buf, int n) {
+  // (LDS is always named through the array itself, so that the compiler knows every such access for what it is:
+  // a read through a plain pointer would wait for the global loads that are under way as well)
+  auto put = [&](int buf, int n) {
 #pragma unroll
     for (int j = 0; j < NHV_DELTA_STAGE; ++j)
-      if (tok_of[j] < n) buf[threadIdx.x + j * n_threads] = hold[j];
+      if (tok_of[j] < n) staged[buf + threadIdx.x + j * n_threads] = hold[j];
   };
   int n_here = min(tile, end - first);
   ask(first, n_here);
-  put(staged, n_here);
+  put(0, n_here);
   __syncthreads();
   int cur = 0;
   for (int t0 = first; t0 < end; t0 += tile) {
     const int n = min(tile, end - t0);
     const int n_next = min(tile, end - t0 - tile);
     if (n_next > 0) ask(t0 + tile, n_next);
-    const float* buf = staged + cur * tile * row;
+    const int buf = cur * tile * row;
+    // a token's vectors are read from LDS into registers while the token before it is computed
+    float nq[DR], nk[DR], ng[DR], nv, nb;
+    auto take = [&](int tok) {
+#pragma unroll
+      for (int i = 0; i < DR; i += 4) {
+        const float4 q4 = *reinterpret_cast<const float4*>(&staged[tok + d0 + i]);
+        const float4 k4 = *reinterpret_cast<const float4*>(&staged[tok + Dp + d0 + i]);
+        const float4 g4 = *reinterpret_cast<const float4*>(&staged[tok + 2 * Dp + d0 + i]);
+        nq[i] = q4.x; nq[i + 1] = q4.y; nq[i + 2] = q4.z; nq[i + 3] = q4.w;
+        nk[i] = k4.x; nk[i + 1] = k4.y; nk[i + 2] = k4.z; nk[i + 3] = k4.w;
+        ng[i] = g4.x; ng[i + 1] = g4.y; ng[i + 2] = g4.z; ng[i + 3] = g4.w;
+      }
+      nv = staged[tok + 3 * Dp + my_col];
+      nb = staged[tok + 3 * Dp + cols];
+    };
+    take(buf);
     for (int i_t = 0; i_t < n; ++i_t) {
-      const float* tok = buf + i_t * row;
       // with S' = diag(g) S:  u = beta (v - k . S'),  o = q . (S' + k u) = q . S' + (q . k) u: the three sums over D are
       // taken together, so a token waits for one exchange between the lanes of its column, not two
       float ck[DR];
       float k_s = 0.f, q_s = 0.f, q_k = 0.f;
+      const float cv = nv, cb = nb;
 #pragma unroll
-      for (int i = 0; i < DR; i += 4) {
-        const float4 q4 = *reinterpret_cast<const float4*>(tok + d0 + i);
-        const float4 k4 = *reinterpret_cast<const float4*>(tok + Dp + d0 + i);
-        const float4 g4 = *reinterpret_cast<const float4*>(tok + 2 * Dp + d0 + i);
-        const float qv[4] = {q4.x, q4.y, q4.z, q4.w}, kv[4] = {k4.x, k4.y, k4.z, k4.w}, gv[4] = {g4.x, g4.y, g4.z, g4.w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          ck[i + j] = kv[j];
-          S[i + j] *= gv[j];
-          k_s = fmaf(kv[j], S[i + j], k_s);
-          q_s = fmaf(qv[j], S[i + j], q_s);
-          q_k = fmaf(qv[j], kv[j], q_k);
-        }
+      for (int i = 0; i < DR; ++i) {
+        ck[i] = nk[i];
+        S[i] *= ng[i];
+        k_s = fmaf(nk[i], S[i], k_s);
+        q_s = fmaf(nq[i], S[i], q_s);
+        q_k = fmaf(nq[i], nk[i], q_k);
       }
-      const float cv = tok[3 * Dp + threadIdx.x / R], cb = tok[3 * Dp + cols];
-      k_s = column_sum(k_s, R);
-      q_s = column_sum(q_s, R);
-      q_k = column_sum(q_k, R);
+      if (i_t + 1 < n) take(buf + (i_t + 1) * row);
+      k_s = column_sum<R>(k_s);
+      q_s = column_sum<R>(q_s);
+      q_k = column_sum<R>(q_k);
       const float u = cb * (cv - k_s);
       const float read = fmaf(q_k, u, q_s);
 #pragma unroll
       for (int i = 0; i < DR; ++i) S[i] = fmaf(ck[i], u, S[i]);
-      if (r == 0 && column) out[((size_t)(t0 + i_t) * H + h) * E + e] = read;
+      if (writes) out_col[(size_t)(t0 + i_t) * H * E] = read;
     }
-    if (n_next > 0) put(staged + (cur ^ 1) * tile * row, n_next);
+    if (n_next > 0) put((cur ^ 1) * tile * row, n_next);
     __syncthreads();
     cur ^= 1;
   }
@@ -323,13 +338,22 @@ extern "C" int nhv_delta_rule(const void* q, const void* k, const void* v, const
   const size_t lds = 2 * (size_t)tile * row * sizeof(float);
   const dim3 grid((E + cols - 1) / cols, H, B), block(n_threads);
   hipStream_t s = (hipStream_t)stream;
-#define LAUNCH(DRV)                                                                                                   \
-  hipLaunchKernelGGL(delta_rule_kernel<DRV>, grid, block, lds, s, (const float*)q, (const float*)k, (const float*)v,  \
+#define LAUNCH(DRV, RV)                                                                                               \
+  hipLaunchKernelGGL((delta_rule_kernel<DRV, RV>), grid, block, lds, s, (const float*)q, (const float*)k, (const float*)v, \
                      (const float*)decay, (const float*)beta, (float*)state, (float*)out, (const int*)positions,      \
-                     (const int*)cu, (const int*)state_slots, H, G, D, E, R, cols, tile)
-  if (dr == 16) LAUNCH(16);
-  else if (dr == 8) LAUNCH(8);
-  else LAUNCH(4);
+                     (const int*)cu, (const int*)state_slots, H, G, D, E, cols, tile)
+#define BY_R(DRV)                          \
+  switch (R) {                             \
+    case 1: LAUNCH(DRV, 1); break;         \
+    case 2: LAUNCH(DRV, 2); break;         \
+    case 4: LAUNCH(DRV, 4); break;         \
+    case 8: LAUNCH(DRV, 8); break;         \
+    case 16: LAUNCH(DRV, 16); break;       \
+    case 32: LAUNCH(DRV, 32); break;       \
+    default: LAUNCH(DRV, 64); break;       \
+  }
+  if (dr == 16) { BY_R(16) } else if (dr == 8) { BY_R(8) } else { BY_R(4) }
+#undef BY_R
 #undef LAUNCH
   NHV_LAUNCH_CHECK("delta_rule");
   return 0;

@@ -68,7 +68,19 @@ CONFIG_R = {
 }
 RANKS_R = {0: (16, 24)}
 
-CASES = {"P": (CONFIG_P, RANKS_P, 11), "Q": (CONFIG_Q, RANKS_Q, 12), "R": (CONFIG_R, RANKS_R, 13)}
+# the same kinds of sizes with chunks longer than a page of 64 tokens, one of them no multiple of it
+CONFIG_S = {
+    "architecture": "Pevazen", "norm": {"eps": 1e-6}, "vocab": 96, "width": 64,
+    "layers": [
+        {"type": "attention", "mlp": _dense(64), "mixer": _attention(4, 1, 32, 32, 96, 16, 10000.0, 0.2)},
+        {"type": "parallel", "mlp": None,
+         "mixer": {"left": _attention(2, 2, 48, 48, 160, 48, 1000.0, 0.15, factor=4.0), "right": _delta(2, 1, 32, 16, 4)}},
+        {"type": "attention", "mlp": _dense(64), "mixer": _attention(4, 1, 32, 32, 128, 16, 10000.0, 0.2, kv_from=0)},
+    ],
+}
+RANKS_S = {1: (8, 8)}
+
+CASES = {"P": (CONFIG_P, RANKS_P, 11), "Q": (CONFIG_Q, RANKS_Q, 12), "R": (CONFIG_R, RANKS_R, 13), "S": (CONFIG_S, RANKS_S, 14)}
 
 
 def random_tensors(config: dict, ranks: dict, seed: int) -> dict[str, torch.Tensor]:

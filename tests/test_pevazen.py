@@ -387,6 +387,19 @@ def test_ways_of_cutting_agree_with_the_plain_model(folders, where, kernels, nam
                 assert torch.equal(results[what][rid], results["whole"][rid]), (what, rid)
 
 
+@pytest.mark.parametrize("where", ON_GPU)
+def test_pages_of_64_and_chunks_longer_than_a_page(folders, where, kernels):
+    """Pages of 64 tokens (whole tiles of the prompt kernel lie in one page) under chunks of 96, 128 and 160
+    positions, requests of up to 400 tokens in portions that end anywhere, beside decoded tokens, on few pages."""
+    device, dtype = where
+    requests = _requests("S", [400, 130, 70, 257])
+    want = _plain_logits(folders["S"], requests)
+    for what, steps in (("portions", pc.in_portions(requests, [37, 2, 64, 5, 1, 129, 1, 1, 96])),
+                        ("side by side", pc.interleaved(requests, [33, 1, 1, 64, 1, 7, 1, 100], 3))):
+        got = _replay(folders["S"], where, steps, page_size=64, max_live=3)
+        _compare(got, want, dtype, what)
+
+
 @pytest.mark.parametrize("where", WHERE)
 def test_long_decoding(folders, where, kernels):
     """Two tokens of prompt, then 140 tokens one by one: the chunks of every layer pass many times, pages go back
@@ -443,3 +456,37 @@ def test_greedy_generation_through_the_entry_point(folders, where, kernels, opti
     stats = llm.get_memory_stats()
     assert stats["live_requests"] == 0 and all(g["free_pages"] == g["pages"] for g in stats["groups"])
     assert stats["state_pool_bytes"] > 0
+
+
+# ------------------------------------------------------------------ the command line
+def _command(*args):
+    import os
+    import subprocess
+    import sys
+    repo = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, "-m", "nanohybrid_vlm_amd", *args], cwd=repo, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    return proc.stdout
+
+
+def test_random_model_of_a_named_shape(tmp_path, emulated_kernels):
+    """``random-model --shape pevazen-tiny`` writes a folder that the plain implementation and the engine both read
+    (its config.json names the two inner sizes that a checkpoint would show by its tensors' shapes)."""
+    out = str(tmp_path / "m")
+    _command("random-model", "--out", out, "--shape", "pevazen-tiny", "--seed", "5")
+    cfg, w = plain.read_model_folder(out)
+    assert cfg["architecture"] == "Pevazen" and w["l0.mix.right.a1"].shape[0] == cfg["layers"][0]["mixer"]["right"]["decay_rank"]
+    requests = {"a": pc.tokens(cfg["vocab"], 31, 1)}
+    want = {"a": plain.logits(cfg, w, requests["a"])}
+    got = _replay(out, CPU, pc.in_portions(requests, [4, 1, 9]), page_size=8, max_live=1)
+    _compare(got, want, "float32", "portions")
+
+
+@pytest.mark.gpu
+def test_generate_command_with_random_weights():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU here")
+    out = json.loads(_command("generate", "--random-weights", "4", "--shape", "pevazen-tiny", "--prompt-ids", "5 17 3",
+                              "--prompt-ids", "9 8 7 6 5 4 3 2 1", "--output-tokens", "6", "--temperature", "0", "--ignore-eos",
+                              "--block-size", "8", "--num-blocks", "32", "--max-model-len", "64", "--quiet"))
+    assert [len(o["token_ids"]) for o in out] == [6, 6]
