@@ -164,7 +164,7 @@ extern "C" int nhv_conv_state_update(const void* proj, int proj_dtype, int ld, v
 // v; beta) come through LDS in tiles of ``tile`` tokens, two buffers: the next tile's loads are under way in registers
 // while this tile is computed, and are stored when it is done; one barrier a tile. A token then costs its
 // arithmetic and two sums over R lanes, not a trip to memory.
-#define NHV_DELTA_STAGE 12     // floats a thread can hold of the next tile (a tile has at most 256 * this many)
+#define NHV_DELTA_STAGE 24     // floats a thread can hold of the next tile (a tile has at most 256 * this many)
 
 // The sum of x over the R adjacent lanes of a column (R a power of two, the groups aligned), in every one of them.
 // Within a row of 16 lanes the partners are reached by lane permutations inside the instruction itself (the two
@@ -183,7 +183,7 @@ __device__ __forceinline__ float column_sum(float x) {
   return x;
 }
 
-template <int DR, int R>
+template <int DR, int R, bool DIRECT>
 __global__ __launch_bounds__(256) void delta_rule_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, const float* __restrict__ decay,
     const float* __restrict__ beta, float* __restrict__ state, float* __restrict__ out, const int* __restrict__ positions,
@@ -207,8 +207,64 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
   float S[DR];
   float* mine = state + (((size_t)state_slots[req] * H + h) * E + (column ? e : 0)) * D;
   const bool fresh = positions[first] == 0;
+  const bool whole4 = (D & 3) == 0;          // (then a lane's entries lie inside D four at a time, and aligned)
 #pragma unroll
-  for (int i = 0; i < DR; ++i) S[i] = (!fresh && column && d0 + i < D) ? mine[d0 + i] : 0.f;
+  for (int i = 0; i < DR; i += 4) {
+    if (whole4) {
+      const float4 s4 = (!fresh && column && d0 + i < D) ? *reinterpret_cast<const float4*>(mine + d0 + i) : float4{0.f, 0.f, 0.f, 0.f};
+      S[i] = s4.x; S[i + 1] = s4.y; S[i + 2] = s4.z; S[i + 3] = s4.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) S[i + j] = (!fresh && column && d0 + i + j < D) ? mine[d0 + i + j] : 0.f;
+    }
+  }
+  if (DIRECT) {
+    // a step of one or two tokens a request (decoding): the token's vectors come straight from memory, this lane's
+    // share of them; nothing goes through LDS and the block meets at no barrier
+    for (int t = first; t < end; ++t) {
+      const float* qr = q + ((size_t)t * G + g) * D;
+      const float* kr = k + ((size_t)t * G + g) * D;
+      const float* gr = decay + ((size_t)t * H + h) * D;
+      float cq[DR], ck[DR];
+      float k_s = 0.f, q_s = 0.f, q_k = 0.f;
+#pragma unroll
+      for (int i = 0; i < DR; i += 4) {
+        float qv[4], kv[4], gv[4];
+        if (whole4 && d0 + i < D) {
+          const float4 q4 = *reinterpret_cast<const float4*>(qr + d0 + i), k4 = *reinterpret_cast<const float4*>(kr + d0 + i),
+                       g4 = *reinterpret_cast<const float4*>(gr + d0 + i);
+          qv[0] = q4.x; qv[1] = q4.y; qv[2] = q4.z; qv[3] = q4.w;
+          kv[0] = k4.x; kv[1] = k4.y; kv[2] = k4.z; kv[3] = k4.w;
+          gv[0] = g4.x; gv[1] = g4.y; gv[2] = g4.z; gv[3] = g4.w;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const bool ok = !whole4 && d0 + i + j < D;
+            qv[j] = ok ? qr[d0 + i + j] : 0.f;
+            kv[j] = ok ? kr[d0 + i + j] : 0.f;
+            gv[j] = ok ? gr[d0 + i + j] : 0.f;
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          cq[i + j] = qv[j];
+          ck[i + j] = kv[j];
+          S[i + j] *= gv[j];
+          k_s = fmaf(kv[j], S[i + j], k_s);
+          q_s = fmaf(qv[j], S[i + j], q_s);
+          q_k = fmaf(qv[j], kv[j], q_k);
+        }
+      }
+      const float cv = column ? v[((size_t)t * H + h) * E + e] : 0.f, cb = beta[(size_t)t * H + h];
+      k_s = column_sum<R>(k_s);
+      q_s = column_sum<R>(q_s);
+      q_k = column_sum<R>(q_k);
+      const float u = cb * (cv - k_s);
+      if (r == 0 && column) out[((size_t)t * H + h) * E + e] = fmaf(q_k, u, q_s);
+#pragma unroll
+      for (int i = 0; i < DR; ++i) S[i] = fmaf(ck[i], u, S[i]);
+    }
+  } else {
 
   // what this thread brings of a tile: entry x of the tile's tile * row floats, x = threadIdx.x + j * n_threads. Which
   // token of the tile and which number of it that is does not change from tile to tile: worked out once.
@@ -308,10 +364,18 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
     __syncthreads();
     cur ^= 1;
   }
+  }
   if (column) {
 #pragma unroll
-    for (int i = 0; i < DR; ++i)
-      if (d0 + i < D) mine[d0 + i] = S[i];
+    for (int i = 0; i < DR; i += 4) {
+      if (whole4) {
+        if (d0 + i < D) *reinterpret_cast<float4*>(mine + d0 + i) = float4{S[i], S[i + 1], S[i + 2], S[i + 3]};
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (d0 + i + j < D) mine[d0 + i + j] = S[i + j];
+      }
+    }
   }
 }
 
@@ -320,8 +384,13 @@ extern "C" int nhv_delta_rule(const void* q, const void* k, const void* v, const
                               int D, int E, int max_q_len, void* stream) {
   NHV_REQUIRE(B > 0 && H > 0 && G > 0 && D > 0 && E > 0 && H % G == 0, "delta_rule: bad sizes B=%d H=%d G=%d D=%d E=%d", B, H, G, D, E);
   NHV_REQUIRE(D <= 1024 && B <= 65535 && H <= 65535, "delta_rule: D=%d (up to 1024), B=%d, H=%d (up to 65535)", D, B, H);
-  // entries a lane: 8 from a key size of 64 on, 4 below, 16 where 8 would need more than 64 lanes a column
-  const int dr = D > 512 ? 16 : (D >= 64 ? 8 : 4);
+  // entries a lane: 4, or what keeps a column within the 64 lanes of a wave. (A token's time is what a wave has to
+  // issue for it, not its arithmetic: 2,048 tokens of 16 heads of 128 x 128 took 890 us with 8 entries a lane and 700 us
+  // with 4, which have one exchange more between the lanes and half the reads from LDS a lane.)
+  // With few requests and heads the chip is far from full and 4 entries a lane are the faster; from about two waves a
+  // SIMD on (4 requests of 2,048 tokens: 1,040 us with 8 entries a lane, 1,450 us with 4) the lanes' own work counts.
+  const long long lanes_at_8 = (long long)B * H * E * ((D + 7) / 8);
+  const int dr = D > 512 ? 16 : ((D > 256 || (D >= 64 && lanes_at_8 >= 100000)) ? 8 : 4);
   int R = 1;
   while (R * dr < D) R <<= 1;
   int cols = 256 / R;
@@ -335,13 +404,19 @@ extern "C" int nhv_delta_rule(const void* q, const void* k, const void* v, const
   if (tile > max_q_len) tile = max_q_len;
   if (tile < 1) tile = 1;
   NHV_REQUIRE(row <= n_threads * NHV_DELTA_STAGE, "delta_rule: a token's %d floats do not fit the block's staging", row);
-  const size_t lds = 2 * (size_t)tile * row * sizeof(float);
+  const bool direct = max_q_len <= 2;
+  const size_t lds = direct ? 0 : 2 * (size_t)tile * row * sizeof(float);
   const dim3 grid((E + cols - 1) / cols, H, B), block(n_threads);
   hipStream_t s = (hipStream_t)stream;
-#define LAUNCH(DRV, RV)                                                                                               \
-  hipLaunchKernelGGL((delta_rule_kernel<DRV, RV>), grid, block, lds, s, (const float*)q, (const float*)k, (const float*)v, \
-                     (const float*)decay, (const float*)beta, (float*)state, (float*)out, (const int*)positions,      \
-                     (const int*)cu, (const int*)state_slots, H, G, D, E, cols, tile)
+#define LAUNCH_AS(DRV, RV, DIR)                                                                                       \
+  hipLaunchKernelGGL((delta_rule_kernel<DRV, RV, DIR>), grid, block, lds, s, (const float*)q, (const float*)k,        \
+                     (const float*)v, (const float*)decay, (const float*)beta, (float*)state, (float*)out,            \
+                     (const int*)positions, (const int*)cu, (const int*)state_slots, H, G, D, E, cols, tile)
+#define LAUNCH(DRV, RV)               \
+  do {                                \
+    if (direct) LAUNCH_AS(DRV, RV, true); \
+    else LAUNCH_AS(DRV, RV, false);   \
+  } while (0)
 #define BY_R(DRV)                          \
   switch (R) {                             \
     case 1: LAUNCH(DRV, 1); break;         \
@@ -355,6 +430,7 @@ extern "C" int nhv_delta_rule(const void* q, const void* k, const void* v, const
   if (dr == 16) { BY_R(16) } else if (dr == 8) { BY_R(8) } else { BY_R(4) }
 #undef BY_R
 #undef LAUNCH
+#undef LAUNCH_AS
   NHV_LAUNCH_CHECK("delta_rule");
   return 0;
 }
