@@ -75,6 +75,9 @@ class ParallelDepthMixBlock(Part):
     feed-forward may be absent."""
 
     norm_slots = ("norm",)
+    # the sum over depth can norm what it hands on in its own kernel: the model names the next block's norm
+    # (``next_norm=``), and that block finds its rows normed already in ``step.scratch``
+    norms_ahead = True
 
     def __init__(self, mixer, feed_forward, norm, depth_index: int, depth_total: int):
         if not 0 <= depth_index < depth_total:
@@ -93,7 +96,7 @@ class ParallelDepthMixBlock(Part):
         n = self.depth_index + 2
         return {"depth.weight": ParamSpec((n,), always_float32=True, init_mean=1.0 / n, init_std=0.3 / n)}
 
-    def forward(self, hidden, residual, step, cache):
+    def forward(self, hidden, residual, step, cache, next_norm=None):
         if residual is not None:
             raise ValueError("this block carries its stream itself and takes no residual beside it")
         if hidden.dtype != torch.float32:
@@ -103,7 +106,16 @@ class ParallelDepthMixBlock(Part):
         if results is None or self.depth_index == 0:
             results = step.scratch["depth_results"] = torch.empty((self.depth_total + 1, T, W), dtype=torch.float32,
                                                                    device=hidden.device)
-        h = self.norm.forward(hidden, out_dtype=self.row_dtype or torch.float32)
+        ahead = step.scratch.pop("normed_ahead", None)
+        if ahead is not None and ahead[0] is self.norm and ahead[1] is hidden:
+            h = ahead[2]                                   # the block before has normed this very stream for this norm
+        else:
+            h = self.norm.forward(hidden, out_dtype=self.row_dtype or torch.float32)
         mixed = self.mixer.forward(h, step, cache)
         fed = self.feed_forward.forward(h, step) if self.feed_forward is not None else None
+        weight, eps = getattr(next_norm, "weight", None), getattr(next_norm, "eps", None)
+        if weight is not None and weight.numel() == 1 and eps is not None and mixed.dtype == (self.row_dtype or torch.float32):
+            out, normed = ops.depth_mix(hidden, mixed, fed, results, self.depth_index, self.depth_weight, gain=weight, eps=eps)
+            step.scratch["normed_ahead"] = (next_norm, out, normed)
+            return out, None
         return ops.depth_mix(hidden, mixed, fed, results, self.depth_index, self.depth_weight), None

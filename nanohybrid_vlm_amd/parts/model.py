@@ -198,6 +198,9 @@ class DecoderModel(Part):
                     nxt = self.layers[order[i + 1].layer]
                     if getattr(nxt, "takes_summed", False):
                         more["next_norm"], more["next_reader"] = nxt.mixer_norm, nxt.mixer
+            elif getattr(layer, "norms_ahead", False) and i + 1 < len(order):
+                # a block that can norm what it hands on for the block that follows: that block's (one) norm
+                more["next_norm"] = getattr(self.layers[order[i + 1].layer], "norm", None)
             hidden, residual = layer.forward(hidden, residual, step, cache, **more)
         if step.num_logit_rows == 0:
             return None
