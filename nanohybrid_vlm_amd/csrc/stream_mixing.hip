@@ -81,19 +81,33 @@ extern "C" int nhv_pair_norm_mean(const void* a, const void* wa, const void* b, 
 // results[0 .. n) are [rows, W] float each, n = index + 2. results[index + 1] = x + (a + b) is written here (and
 // results[0] = x when index is 0: the stream that enters the first layer is the first result); then
 // out = sum over j < n of weights[j] * results[j], in rising j. With ``gain`` the RMS norm of out with that one number
-// as its weight is written to ``normed`` as well (what the next layer reads).
+// as its weight is written to ``normed`` as well (what the next layer reads). With ``a2`` the first addend is not a but
+// half the sum of a and a2, each over its root mean square (pair_eps) times its weight vector wa, wb: what
+// nhv_pair_norm_mean would have written, unrounded.
 template <typename T>
 __global__ void depth_mix_kernel(const float* __restrict__ x, const T* __restrict__ a, const T* __restrict__ b,
                                  float* __restrict__ results, size_t plane, int index, const float* __restrict__ weights,
                                  float* __restrict__ out, const float* __restrict__ gain, T* __restrict__ normed, int W,
-                                 float eps) {
+                                 float eps, const T* __restrict__ a2, const float* __restrict__ wa,
+                                 const float* __restrict__ wb, float pair_eps) {
   __shared__ float scratch[16];
   const size_t base = (size_t)blockIdx.x * W;
   const int n = index + 2;
+  float ra = 1.f, rb = 0.f;
+  if (a2 != nullptr) {
+    float sa = 0.f, sb = 0.f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+      const float u = to_f32(a[base + i]), v = to_f32(a2[base + i]);
+      sa = fmaf(u, u, sa);
+      sb = fmaf(v, v, sb);
+    }
+    ra = 1.0f / sqrtf(block_sum(sa, scratch) / (float)W + pair_eps);
+    rb = 1.0f / sqrtf(block_sum(sb, scratch) / (float)W + pair_eps);
+  }
   float ss = 0.f;
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
     const float xi = x[base + i];
-    float add = to_f32(a[base + i]);
+    float add = a2 != nullptr ? 0.5f * (to_f32(a[base + i]) * ra * wa[i] + to_f32(a2[base + i]) * rb * wb[i]) : to_f32(a[base + i]);
     if (b != nullptr) add += to_f32(b[base + i]);
     const float mine = xi + add;
     results[(size_t)(index + 1) * plane + base + i] = mine;
@@ -112,18 +126,19 @@ __global__ void depth_mix_kernel(const float* __restrict__ x, const T* __restric
 
 extern "C" int nhv_depth_mix(const void* x, const void* a, const void* b, void* results, long long plane, int index,
                              const void* weights, void* out, const void* gain, void* normed, int T, int W, float eps,
-                             int dtype, void* stream) {
+                             const void* a2, const void* wa, const void* wb, float pair_eps, int dtype, void* stream) {
   NHV_REQUIRE(T > 0 && W > 0 && index >= 0 && plane >= (long long)T * W, "depth_mix: bad sizes T=%d W=%d index=%d", T, W, index);
   NHV_REQUIRE(x != out, "depth_mix: the sum cannot be written over the stream it reads");
+  NHV_REQUIRE(a2 == nullptr || (wa != nullptr && wb != nullptr), "depth_mix: a pair of addends without its weights");
   hipStream_t s = (hipStream_t)stream;
   if (dtype == NHV_F32)
     hipLaunchKernelGGL(depth_mix_kernel<float>, dim3(T), dim3(256), 0, s, (const float*)x, (const float*)a, (const float*)b,
                        (float*)results, (size_t)plane, index, (const float*)weights, (float*)out, (const float*)gain,
-                       (float*)normed, W, eps);
+                       (float*)normed, W, eps, (const float*)a2, (const float*)wa, (const float*)wb, pair_eps);
   else if (dtype == NHV_BF16)
     hipLaunchKernelGGL(depth_mix_kernel<bf16_t>, dim3(T), dim3(256), 0, s, (const float*)x, (const bf16_t*)a, (const bf16_t*)b,
                        (float*)results, (size_t)plane, index, (const float*)weights, (float*)out, (const float*)gain,
-                       (bf16_t*)normed, W, eps);
+                       (bf16_t*)normed, W, eps, (const bf16_t*)a2, (const float*)wa, (const float*)wb, pair_eps);
   else return nhv_fail("depth_mix: unknown dtype %d", dtype);
   NHV_LAUNCH_CHECK("depth_mix");
   return 0;

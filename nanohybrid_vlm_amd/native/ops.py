@@ -206,10 +206,12 @@ class NativeBackend:
         self._call("nhv_pair_norm_mean", _ptr(a), _ptr(wa), _ptr(b), _ptr(wb), _ptr(y), T, W, ctypes.c_float(eps),
                    dtype_code(a), _stream())
 
-    def depth_mix(self, x, a, b, results, index, weights, out, gain, normed, eps):
+    def depth_mix(self, x, a, b, results, index, weights, out, gain, normed, eps, pair=None):
         T, W = x.shape
+        a2, wa, wb, pair_eps = pair if pair is not None else (None, None, None, 0.0)
         self._call("nhv_depth_mix", _ptr(x), _ptr(a), _ptr(b), _ptr(results), ctypes.c_longlong(results.stride(0)), index,
-                   _ptr(weights), _ptr(out), _ptr(gain), _ptr(normed), T, W, ctypes.c_float(eps), dtype_code(a), _stream())
+                   _ptr(weights), _ptr(out), _ptr(gain), _ptr(normed), T, W, ctypes.c_float(eps), _ptr(a2), _ptr(wa),
+                   _ptr(wb), ctypes.c_float(pair_eps), dtype_code(a), _stream())
 
     def rotary_split_write(self, qkv, bias, qk_freqs, rot, v_freqs, positions, slot_mapping, q_out, k_cache, v_cache,
                            Hq, Hkv, D, E, with_kv):
@@ -740,6 +742,8 @@ def dense(x):
         return x.tensor()
     if isinstance(x, Summed):
         raise KernelError("a sum that was made for a norm (ops.Summed) goes through that norm, not anywhere else")
+    if isinstance(x, NormedPairMean):
+        return x.tensor()
     return x
 
 
@@ -1025,14 +1029,37 @@ def pair_norm_mean(a: torch.Tensor, wa: torch.Tensor, b: torch.Tensor, wb: torch
     return y
 
 
-def depth_mix(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor | None, results: torch.Tensor, index: int,
+@dataclass
+class NormedPairMean:
+    """Half the sum of two rows' norms (each over its root mean square, times a weight vector of its own) that is
+    still to be taken: ``depth_mix`` takes it as its first addend and does the work in its own kernel; ``tensor()``
+    is the same as a tensor (``pair_norm_mean``), for any other reader."""
+
+    a: torch.Tensor
+    wa: torch.Tensor
+    b: torch.Tensor
+    wb: torch.Tensor
+    eps: float
+
+    def tensor(self) -> torch.Tensor:
+        return pair_norm_mean(self.a, self.wa, self.b, self.wb, self.eps)
+
+
+def depth_mix(x: torch.Tensor, a, b: torch.Tensor | None, results: torch.Tensor, index: int,
               weights: torch.Tensor, gain: torch.Tensor | None = None, eps: float = 0.0):
     """results[index + 1] = x + (a + b) (and results[0] = x when ``index`` is 0); returns the float32 stream
     sum over j <= index + 1 of weights[j] * results[j], and with ``gain`` also its RMS norm (one number as weight)
-    in the element type of ``a``. ``x``: [tokens, width] float32; ``results``: [depth, tokens, width] float32."""
+    in the element type of ``a``. ``x``: [tokens, width] float32; ``results``: [depth, tokens, width] float32.
+    ``a`` may be a ``NormedPairMean``."""
     _need(x.dim() == 2, "depth_mix: x must be [tokens, width]")
     T, W = x.shape
     _dense(x, "depth_mix: x", dtype=torch.float32)
+    pair = None
+    if isinstance(a, NormedPairMean):
+        _dense(a.b, "depth_mix: the pair's second rows", (T, W), a.a.dtype)
+        _float_vector(a.wa, "depth_mix: the pair's first weight", (W,))
+        _float_vector(a.wb, "depth_mix: the pair's second weight", (W,))
+        pair, a = (a.b, a.wa, a.wb, float(a.eps)), a.a
     _dense(a, "depth_mix: a", (T, W))
     dtype_code(a)
     if b is not None:
@@ -1047,7 +1074,7 @@ def depth_mix(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor | None, results:
         _need(gain.numel() == 1, "depth_mix: the norm's weight is one number")
         _dense(gain, "depth_mix: norm weight", dtype=torch.float32)
         normed = torch.empty((T, W), dtype=a.dtype, device=a.device)
-    backend().depth_mix(x, a, b, results, int(index), weights, out, gain, normed, float(eps))
+    backend().depth_mix(x, a, b, results, int(index), weights, out, gain, normed, float(eps), **({"pair": pair} if pair else {}))
     return (out, normed) if gain is not None else out
 
 

@@ -111,10 +111,12 @@ class ParallelDepthMixBlock(Part):
             h = ahead[2]                                   # the block before has normed this very stream for this norm
         else:
             h = self.norm.forward(hidden, out_dtype=self.row_dtype or torch.float32)
-        mixed = self.mixer.forward(h, step, cache)
+        # (a pair of mixers may leave its two norms and their mean to the sum over depth)
+        mixed = self.mixer.forward(h, step, cache, **({"deferred": True} if getattr(self.mixer, "defers_pair_norm", False) else {}))
         fed = self.feed_forward.forward(h, step) if self.feed_forward is not None else None
         weight, eps = getattr(next_norm, "weight", None), getattr(next_norm, "eps", None)
-        if weight is not None and weight.numel() == 1 and eps is not None and mixed.dtype == (self.row_dtype or torch.float32):
+        rows = mixed.a if isinstance(mixed, ops.NormedPairMean) else mixed
+        if weight is not None and weight.numel() == 1 and eps is not None and rows.dtype == (self.row_dtype or torch.float32):
             out, normed = ops.depth_mix(hidden, mixed, fed, results, self.depth_index, self.depth_weight, gain=weight, eps=eps)
             step.scratch["normed_ahead"] = (next_norm, out, normed)
             return out, None

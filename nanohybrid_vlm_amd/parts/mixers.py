@@ -234,7 +234,12 @@ class NormedPair(Part):
                 state = need
         return CombinedNeed(paged, state)
 
-    def forward(self, x, step, cache: CacheView):
+    defers_pair_norm = True       # ``forward(..., deferred=True)`` may return an ``ops.NormedPairMean``
+
+    def forward(self, x, step, cache: CacheView, deferred: bool = False):
+        """``deferred``: the caller's next step is a kernel that takes the two results with their norms still to do
+        (``ops.depth_mix``); it then gets an ``ops.NormedPairMean`` in place of a tensor."""
         a = self.left.forward(x, step, cache)
         b = self.right.forward(x, step, cache)
-        return ops.pair_norm_mean(a, self.left_out_weight, b, self.right_out_weight, self.eps)
+        pair = ops.NormedPairMean(a, self.left_out_weight, b, self.right_out_weight, self.eps)
+        return pair if deferred else pair.tensor()

@@ -109,8 +109,14 @@ class EmulatedBackend:
             return t / torch.sqrt(t.pow(2).mean(-1, keepdim=True) + eps) * w
         y.copy_((0.5 * (norm(a, wa) + norm(b, wb))).to(y.dtype))
 
-    def depth_mix(self, x, a, b, results, index, weights, out, gain, normed, eps):
-        add = a.float() if b is None else a.float() + b.float()
+    def depth_mix(self, x, a, b, results, index, weights, out, gain, normed, eps, pair=None):
+        add = a.float()
+        if pair is not None:
+            a2, wa, wb, pair_eps = pair
+            unit = lambda t: t.float() / torch.sqrt(t.float().pow(2).mean(-1, keepdim=True) + pair_eps)
+            add = 0.5 * (unit(a) * wa + unit(a2) * wb)
+        if b is not None:
+            add = add + b.float()
         if index == 0:
             results[0] = x
         results[index + 1] = x + add

@@ -105,6 +105,15 @@ def test_norms_and_depth_sum(where, kernels):
         stream = got.cpu()
     with pytest.raises(ops.KernelError):
         ops.depth_mix(x.to(device), a.to(device), None, results, depth, torch.ones(depth + 2).to(device))
+    # a pair of rows whose norms and mean are left to the sum over depth, with the next norm taken in the same kernel
+    pair = ops.NormedPairMean(a.to(device), wa.to(device), b.to(device), wb.to(device), eps)
+    w = torch.tensor([0.3, 0.9])
+    got, normed = ops.depth_mix(x.to(device), pair, b.to(device), results, 0, w.to(device), gain=gain.to(device), eps=eps)
+    mean = 0.5 * (plain.vector_norm(a.float(), wa, eps) + plain.vector_norm(b.float(), wb, eps))
+    want = w[0] * x + w[1] * (x + (mean + b.float()))
+    assert max_abs_diff(got.cpu(), want) <= 1e-5 * float(want.abs().max())
+    assert max_abs_diff(normed.float().cpu(), plain.scalar_norm(want, gain, eps)) <= _tol(dtype, want)
+    assert max_abs_diff(pair.tensor().float().cpu(), mean) <= _tol(dtype, mean)
 
 
 def _attention_through_kernels(device, dtype, m, q_in, k_in, v_in, portions, page_size, rotate_values, bias=None):
