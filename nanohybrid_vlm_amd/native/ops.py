@@ -997,7 +997,8 @@ def gated_linear(x, w: torch.Tensor) -> torch.Tensor:
 
 
 # ------------------------------------------------------------------ layers that are not the pre-norm kind
-def _float_vector(t: torch.Tensor, name: str, shape: tuple) -> None:
+def _float32(t: torch.Tensor, name: str, shape: tuple) -> None:
+    """A dense float32 tensor of this shape (weights and statistics that stay in 32-bit whatever the rows are)."""
     _dense(t, name, shape, torch.float32)
 
 
@@ -1021,8 +1022,8 @@ def pair_norm_mean(a: torch.Tensor, wa: torch.Tensor, b: torch.Tensor, wb: torch
     _need(a.dim() == 2, "pair_norm_mean: rows must be [tokens, width]")
     _dense(a, "pair_norm_mean: a")
     _dense(b, "pair_norm_mean: b", tuple(a.shape), a.dtype)
-    _float_vector(wa, "pair_norm_mean: first weight", (a.shape[1],))
-    _float_vector(wb, "pair_norm_mean: second weight", (a.shape[1],))
+    _float32(wa, "pair_norm_mean: first weight", (a.shape[1],))
+    _float32(wb, "pair_norm_mean: second weight", (a.shape[1],))
     dtype_code(a)
     y = torch.empty_like(a)
     backend().pair_norm_mean(a, wa, b, wb, y, float(eps))
@@ -1057,8 +1058,8 @@ def depth_mix(x: torch.Tensor, a, b: torch.Tensor | None, results: torch.Tensor,
     pair = None
     if isinstance(a, NormedPairMean):
         _dense(a.b, "depth_mix: the pair's second rows", (T, W), a.a.dtype)
-        _float_vector(a.wa, "depth_mix: the pair's first weight", (W,))
-        _float_vector(a.wb, "depth_mix: the pair's second weight", (W,))
+        _float32(a.wa, "depth_mix: the pair's first weight", (W,))
+        _float32(a.wb, "depth_mix: the pair's second weight", (W,))
         pair, a = (a.b, a.wa, a.wb, float(a.eps)), a.a
     _dense(a, "depth_mix: a", (T, W))
     dtype_code(a)
@@ -1067,7 +1068,7 @@ def depth_mix(x: torch.Tensor, a, b: torch.Tensor | None, results: torch.Tensor,
     _need(results.dim() == 3 and tuple(results.shape[1:]) == (T, W) and 0 <= index and index + 2 <= results.shape[0],
           lambda: f"depth_mix: results {tuple(results.shape)} for index {index} and rows {(T, W)}")
     _dense(results, "depth_mix: results", dtype=torch.float32)
-    _float_vector(weights, "depth_mix: weights", (index + 2,))
+    _float32(weights, "depth_mix: weights", (index + 2,))
     out = torch.empty_like(x)
     normed = None
     if gain is not None:
@@ -1095,7 +1096,7 @@ def rotary_split_write(qkv: torch.Tensor, bias: torch.Tensor | None, qk_freqs: t
     if qk_freqs is not None:
         rot = 2 * qk_freqs.shape[0]
         _need(rot <= head_dim, lambda: f"rotary_split_write: rotary size {rot} with head size {head_dim}")
-        _float_vector(qk_freqs, "rotary_split_write: frequencies", (rot // 2,))
+        _float32(qk_freqs, "rotary_split_write: frequencies", (rot // 2,))
     _dense(positions, "rotary_split_write: positions", (T,), torch.int32)
     if with_kv:
         _dense(slot_mapping, "rotary_split_write: slot_mapping", (T,), torch.int32)
@@ -1107,7 +1108,7 @@ def rotary_split_write(qkv: torch.Tensor, bias: torch.Tensor | None, qk_freqs: t
         _dense(v_cache, "rotary_split_write: v_cache", dtype=qkv.dtype)
         if v_freqs is not None:
             _need(value_dim % 2 == 0, "rotary_split_write: value heads of odd size cannot be turned")
-            _float_vector(v_freqs, "rotary_split_write: value frequencies", (value_dim // 2,))
+            _float32(v_freqs, "rotary_split_write: value frequencies", (value_dim // 2,))
     q_out = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
     if T:
         backend().rotary_split_write(qkv, bias, qk_freqs, rot, v_freqs if with_kv else None, positions,
@@ -1121,7 +1122,7 @@ def turn_back_(x: torch.Tensor, freqs: torch.Tensor, positions: torch.Tensor) ->
     _need(x.dim() == 3 and x.shape[2] % 2 == 0, "turn_back: x must be [tokens, heads, even size]")
     _dense(x, "turn_back: x")
     dtype_code(x)
-    _float_vector(freqs, "turn_back: frequencies", (x.shape[2] // 2,))
+    _float32(freqs, "turn_back: frequencies", (x.shape[2] // 2,))
     _dense(positions, "turn_back: positions", (x.shape[0],), torch.int32)
     if x.shape[0]:
         backend().turn_back(x, freqs, positions)
@@ -1145,15 +1146,15 @@ def gated_delta_rule(proj: torch.Tensor, a_lin: torch.Tensor, gate_lin: torch.Te
     _need(H % G == 0, lambda: f"gated_delta_rule: {H} heads are not a multiple of {G} key heads")
     _dense(proj, "gated_delta_rule: proj", (T, C + H))
     dtype_code(proj)
-    _float_vector(a_lin, "gated_delta_rule: decays' linear part", (T, H * D))
-    _float_vector(gate_lin, "gated_delta_rule: gates' linear part", (T, H * E))
+    _float32(a_lin, "gated_delta_rule: decays' linear part", (T, H * D))
+    _float32(gate_lin, "gated_delta_rule: gates' linear part", (T, H * E))
     _need(taps.dim() == 2 and taps.shape[0] == C and 1 <= taps.shape[1] <= 16,
           lambda: f"gated_delta_rule: taps {tuple(taps.shape)} for {C} channels (1 to 16 taps)")
     _dense(taps, "gated_delta_rule: taps", dtype=torch.float32)
     n = taps.shape[1]
-    _float_vector(dt_bias, "gated_delta_rule: dt_bias", (H * D,))
-    _float_vector(a_log, "gated_delta_rule: a_log", (H,))
-    _float_vector(norm_weight, "gated_delta_rule: norm weight", (E,))
+    _float32(dt_bias, "gated_delta_rule: dt_bias", (H * D,))
+    _float32(a_log, "gated_delta_rule: a_log", (H,))
+    _float32(norm_weight, "gated_delta_rule: norm weight", (E,))
     _need(kept.dim() == 3 and tuple(kept.shape[1:]) == (C, n - 1), lambda: f"gated_delta_rule: kept inputs {tuple(kept.shape)}")
     _dense(kept, "gated_delta_rule: kept inputs", dtype=torch.float32)
     _need(state.dim() == 4 and tuple(state.shape[1:]) == (H, E, D) and state.shape[0] == kept.shape[0],

@@ -5,7 +5,6 @@ slots that are used again), and greedy generation through the entry point and it
 the CPU stand-in for the kernels (the engine's logic) and, marked ``gpu``, on the HIP kernels in both element types.
 """
 import json
-import math
 
 import pytest
 import torch
@@ -499,3 +498,27 @@ def test_generate_command_with_random_weights():
                               "--prompt-ids", "9 8 7 6 5 4 3 2 1", "--output-tokens", "6", "--temperature", "0", "--ignore-eos",
                               "--block-size", "8", "--num-blocks", "32", "--max-model-len", "64", "--quiet"))
     assert [len(o["token_ids"]) for o in out] == [6, 6]
+
+
+# ------------------------------------------------------------------ the replay program
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_program_on_a_model_of_this_design(folders, dtype, tmp_path):
+    """``bin/trace_run`` as a user starts it: steps on standard input, ``<step>.f32`` files, pages of 64 and four
+    state slots that several traces in one run use again, steps of single tokens and short mixed steps from graphs."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU here")
+    from test_replay import _logits_from_files, _renamed, _trace_run
+    requests = _requests("S", [150, 9, 71, 2, 40])
+    want = _plain_logits(folders["S"], requests)
+    ways = {"portions": pc.in_portions(requests, [37, 2, 64, 5, 1, 1]),
+            "side by side": pc.interleaved(requests, [33, 1, 1, 16, 1, 7, 1], 4)}
+    steps, first = [], 0
+    for k, (what, t) in enumerate(ways.items()):
+        steps += _renamed(t, f"#{k}", first)
+        first += len(t)
+    out_dir = str(tmp_path / "out")
+    _trace_run(folders["S"], dtype, steps, out_dir, max(pc.peak_tokens(t, 64) for t in ways.values()))
+    got = _logits_from_files(out_dir, steps, pc.CONFIG_S["vocab"])
+    for k, what in enumerate(ways):
+        _compare({rid: got[f"{rid}#{k}"] for rid in want}, want, dtype, what)
