@@ -155,7 +155,8 @@ class ModelRunner:
         if not windows:
             windows = [(None, None)]                   # a model without paged layers still has one (empty) group
         self._windows = windows
-        if self.share_prefixes and any(_state(n) is not None for n in needs):
+        embedding_need = self.model.embedding_state_need()
+        if self.share_prefixes and (embedding_need is not None or any(_state(n) is not None for n in needs)):
             # state of fixed size summarises all earlier tokens: pages alone do not bring a prefix back
             # (the reference switches the page hashes off for such models, nanovllm/config.py:384-399)
             raise ValueError("prefixes cannot be shared by a model with per-request state")
@@ -171,8 +172,15 @@ class ModelRunner:
                         for name, (shape, dt) in _state(need).tensors.items()}
                 self.state_pools.append(pool)
                 self._state_views[i] = CacheView(kind="state", state=pool)
+        if embedding_need is not None:
+            # what the embedding keeps per request is one more pool: recorded steps and steps issued ahead put its
+            # rows back as they do every other pool's
+            pool = {name: torch.zeros((num_state_slots + 1, *shape), dtype=dt, device=self.device)
+                    for name, (shape, dt) in embedding_need.tensors.items()}
+            self.state_pools.append(pool)
+            self.model.attach_embedding_state(pool)
         item = torch.empty((), dtype=self.dtype).element_size()
-        page_bytes = sum(page_size * n.num_kv_heads * (n.head_dim + n.value_size) * item
+        page_bytes = sum(page_size * n.num_kv_heads * n.stored_per_head * item
                          for n in map(_paged, needs) if n is not None)
         if num_pages is None:
             num_pages = self._pages_from_free_memory(page_bytes, utilization, max_tokens)
@@ -196,7 +204,13 @@ class ModelRunner:
                 # (nanovllm/engine/model_runner.py:870-906). The last page is handed to no request and holds zeros:
                 # the padding rows of a recorded step read their one key there. Value heads of another size than
                 # the key heads get a tensor of their own.
-                if need.value_size == need.head_dim:
+                if need.values_in_keys:
+                    # one row a token and head, read as key and as value
+                    k = torch.empty((num_pages + 1, page_size, need.num_kv_heads, need.head_dim), dtype=self.dtype, device=self.device)
+                    k[num_pages].zero_()
+                    v = k
+                    self.kv_tensors.append(k[:num_pages])
+                elif need.value_size == need.head_dim:
                     kv = torch.empty((2, num_pages + 1, page_size, need.num_kv_heads, need.head_dim),
                                      dtype=self.dtype, device=self.device)
                     kv[:, num_pages].zero_()

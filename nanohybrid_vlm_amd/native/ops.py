@@ -19,7 +19,8 @@ import torch
 from . import library
 
 CORE_SOURCES = ["error.hip", "elementwise.hip", "gemm_generic.hip", "gemm_skinny_bf16.hip", "gemm_fewrows_bf16.hip", "attention_generic.hip",
-                "sampling.hip", "measure.hip", "stream_mixing.hip", "delta_rule.hip"]
+                "sampling.hip", "measure.hip", "stream_mixing.hip", "delta_rule.hip", "parallel_block.hip", "latent_attention.hip",
+                "routed_experts.hip"]
 BLAS_SOURCES = ["error.hip", "gemm_library.hip"]                                                   # the vendor's matrix library, algorithm by number
 BLAS_LINK = ["-lhipblaslt"]
 ATTENTION_SOURCES = ["error.hip", "attention_decode_bf16.hip", "attention_prefill_bf16.hip"]      # compiled once per head size
@@ -245,6 +246,72 @@ class NativeBackend:
         T, H, E = o.shape
         self._call("nhv_gated_head_norm", _ptr(o), _ptr(gate), _ptr(w), _ptr(y), T, H, E, ctypes.c_float(eps),
                    dtype_code(y), _stream())
+
+    # -- layers of two norms side by side, an embedding with a hashed pair row --
+    def embed_pair_hash(self, ids, table, pair_table, out, batch, state_slots, prev_state, buckets, mul_prev, mul_cur):
+        T, W = out.shape
+        self._call("nhv_embed_pair_hash", _ptr(ids), _ptr(table), _ptr(pair_table), _ptr(out), _ptr(batch.positions),
+                   _ptr(batch.cu_seqlens_q), _ptr(batch.token_req), _ptr(state_slots), _ptr(prev_state), T, W,
+                   table.shape[0], buckets, mul_prev, mul_cur, dtype_code(table), _stream())
+
+    def layernorm_pair(self, x, a, b, w1, b1, y1, w2, b2, y2, eps, rows_dtype):
+        T, W = x.shape
+        self._call("nhv_layernorm_pair", _ptr(x), _ptr(a), _ptr(b), _ptr(w1), _ptr(b1), _ptr(y1), _ptr(w2), _ptr(b2),
+                   _ptr(y2), T, W, ctypes.c_float(eps), _DTYPE_CODE[rows_dtype], _stream())
+
+    def add_streams(self, x, a, b):
+        self._call("nhv_add_streams", _ptr(x), _ptr(a), _ptr(b), ctypes.c_size_t(x.numel()), dtype_code(a), _stream())
+
+    def act_mul(self, gu, out, act):
+        T, I = out.shape
+        self._call("nhv_act_mul", _ptr(gu), _ptr(out), T, I, act, dtype_code(gu), _stream())
+
+    # -- attention over a cached latent --
+    def latent_prepare(self, a, q_off, q_rank, c_off, kv_rank, rot, wq, wc, eps, freqs, gain, positions, slot_mapping,
+                       cache, cq):
+        self._call("nhv_latent_prepare", _ptr(a), a.shape[1], q_off, q_rank, c_off, kv_rank, rot, _ptr(wq), _ptr(wc),
+                   ctypes.c_float(eps), _ptr(freqs), ctypes.c_float(gain), _ptr(positions), _ptr(slot_mapping), _ptr(cache),
+                   0 if cache is None else cache.shape[-1], _ptr(cq), a.shape[0], dtype_code(cq), _stream())
+
+    def head_gemm(self, x, x_off, x_row, w, w_head, w_n, w_k, y, y_off, y_row, gate, gate_off, N, K):
+        """y[t, h, y_off : y_off + N] = M_h x[t, h, x_off : x_off + K]; x and y are [rows, heads, x_row / y_row]."""
+        T, H = x.shape[0], x.shape[1]
+        item = x.element_size()
+        LL = ctypes.c_longlong
+        gate_p = None if gate is None else ctypes.c_void_p(gate.data_ptr() + 4 * gate_off)
+        if x.dtype == torch.bfloat16 and T > self.few_rows and not self.own_kernels_only and gate is None:
+            # many rows: the library's batched product, one matrix per head, on strided views
+            xv = x[:, :, x_off:x_off + K].transpose(0, 1)                         # [H, T, K]
+            wv = torch.as_strided(w, (H, K, N), (w_head, w_k, w_n))
+            yv = y[:, :, y_off:y_off + N].transpose(0, 1)
+            yv.copy_(torch.bmm(xv, wv))
+            return
+        self._call("nhv_head_gemm", ctypes.c_void_p(x.data_ptr() + item * x_off), LL(H * x_row), LL(x_row), _ptr(w),
+                   LL(w_head), LL(w_n), LL(w_k), ctypes.c_void_p(y.data_ptr() + item * y_off), LL(H * y_row), LL(y_row),
+                   gate_p, LL(0 if gate is None else gate.shape[1]), T, H, N, K, dtype_code(x), _stream())
+
+    def rotate_interleaved(self, src, s_off, dst, d_off, rot, freqs, gain, positions):
+        T, H, s_row = src.shape
+        self._call("nhv_rotate_interleaved", _ptr(src), s_row, s_off, _ptr(dst), dst.shape[2], d_off, rot, _ptr(freqs),
+                   ctypes.c_float(gain), _ptr(positions), T, H, dtype_code(src), _stream())
+
+    # -- a feed-forward of many small experts --
+    def route_topk(self, h, router, ids, scores):
+        T, W = h.shape
+        self._call("nhv_route_topk", _ptr(h), _ptr(router), _ptr(ids), _ptr(scores), T, W, router.shape[0], ids.shape[1],
+                   dtype_code(h), _stream())
+
+    def experts_gate_up(self, h, ids, scores, gate_up, u, act):
+        T, W = h.shape
+        E, F2, _ = gate_up.shape
+        self._call("nhv_experts_gate_up", _ptr(h), _ptr(ids), _ptr(scores), _ptr(gate_up), _ptr(u), T, W, F2 // 2,
+                   ids.shape[1], E, act, dtype_code(h), _stream())
+
+    def experts_down(self, u, ids, down, out):
+        T, W = out.shape
+        E, _, F = down.shape
+        self._call("nhv_experts_down", _ptr(u), _ptr(ids), _ptr(down), _ptr(out), T, W, F, ids.shape[1], E,
+                   dtype_code(u), _stream())
 
     def _decode_attention(self, q, k_cache, v_cache, out, batch, block_tables, scale, window):
         """Single tokens in bfloat16: keys split over waves, then merged."""
@@ -995,6 +1062,205 @@ def gated_linear(x, w: torch.Tensor) -> torch.Tensor:
             return out
     return silu_mul(linear(x, w))
 
+
+
+# ------------------------------------------------------------------ two norms side by side, a hashed pair embedding
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def embed_pair_hash(ids: torch.Tensor, table: torch.Tensor, pair_table: torch.Tensor, batch: AttentionBatch,
+                    state_slots: torch.Tensor, prev_state: torch.Tensor, buckets: int, mul_prev: int, mul_cur: int) -> torch.Tensor:
+    """float32 [tokens, width]: table[id] + pair_table[(previous id * mul_prev + id * mul_cur) mod buckets], and for a
+    token at position 0 the row ``buckets``. The id before a portion's first token is ``prev_state`` at the request's
+    slot ([slots] int32), which then takes the portion's last id."""
+    T = ids.shape[0]
+    _need(table.dim() == 2 and pair_table.dim() == 2 and pair_table.shape[1] == table.shape[1],
+          "embed_pair_hash: tables must be [rows, width] of one width")
+    _dense(table, "embed_pair_hash: table")
+    _dense(pair_table, "embed_pair_hash: pair table", dtype=table.dtype)
+    _need(buckets > 0 and pair_table.shape[0] == buckets + 1,
+          lambda: f"embed_pair_hash: a pair table of {pair_table.shape[0]} rows for {buckets} buckets and one row more")
+    _dense(ids, "embed_pair_hash: ids", (T,), torch.int32)
+    _need(T == batch.num_tokens, lambda: f"embed_pair_hash: {T} tokens but the batch has {batch.num_tokens}")
+    _dense(batch.positions, "embed_pair_hash: positions", (T,), torch.int32)
+    _dense(batch.token_req, "embed_pair_hash: token_req", (T,), torch.int32)
+    _dense(batch.cu_seqlens_q, "embed_pair_hash: cu_seqlens_q", (batch.num_requests + 1,), torch.int32)
+    _dense(state_slots, "embed_pair_hash: state_slots", (batch.num_requests,), torch.int32)
+    _need(prev_state.dim() == 1, "embed_pair_hash: the kept tokens are one number a slot")
+    _dense(prev_state, "embed_pair_hash: prev_state", dtype=torch.int32)
+    dtype_code(table)
+    out = torch.empty((T, table.shape[1]), dtype=torch.float32, device=table.device)
+    backend().embed_pair_hash(ids, table, pair_table, out, batch, state_slots, prev_state, int(buckets), int(mul_prev), int(mul_cur))
+    return out
+
+
+def layernorm_pair(x: torch.Tensor, first, second, eps: float, out_dtype, add=()):
+    """Layer norms (weight and bias, float32) of the float32 stream ``x``, one per (weight, bias) given: ``first`` and
+    ``second`` (either may be None). ``add``: up to two tensors of rows that are added to ``x`` first, in float, in
+    place. Mean and variance are taken once. Returns (y1 or None, y2 or None) in ``out_dtype``."""
+    _need(x.dim() == 2, "layernorm_pair: x must be [tokens, width]")
+    _dense(x, "layernorm_pair: x", dtype=torch.float32)
+    W = x.shape[1]
+    add = [t for t in add if t is not None]
+    _need(len(add) <= 2, "layernorm_pair: at most two tensors are added")
+    for t in add:
+        _dense(t, "layernorm_pair: an added tensor", tuple(x.shape), out_dtype)
+    _need(out_dtype in _DTYPE_CODE, lambda: f"layernorm_pair: rows of {out_dtype}")
+    outs, args = [], []
+    for wb in (first, second):
+        if wb is None:
+            outs.append(None)
+            args += [None, None, None]
+            continue
+        w, b = wb
+        _float32(w, "layernorm_pair: weight", (W,))
+        _float32(b, "layernorm_pair: bias", (W,))
+        y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        outs.append(y)
+        args += [w, b, y]
+    _need(outs[0] is not None or outs[1] is not None or add, "layernorm_pair: nothing to do")
+    a = add[0] if add else None
+    b = add[1] if len(add) > 1 else None
+    backend().layernorm_pair(x, a, b, *args, float(eps), out_dtype)
+    return outs[0], outs[1]
+
+
+def add_streams_(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor | None = None) -> torch.Tensor:
+    """x += a (+ b) in float, in place; x is the float32 stream."""
+    _dense(x, "add_streams: x", dtype=torch.float32)
+    _dense(a, "add_streams: a", tuple(x.shape))
+    dtype_code(a)
+    if b is not None:
+        _dense(b, "add_streams: b", tuple(x.shape), a.dtype)
+    backend().add_streams(x, a, b)
+    return x
+
+
+def act_mul(gate_up: torch.Tensor, activation: str) -> torch.Tensor:
+    """act(gate) * up for rows [gate | up]; ``activation``: "silu" or "gelu_tanh"."""
+    _need(activation in ACTIVATIONS, lambda: f"act_mul: activation {activation!r} is not known ({sorted(ACTIVATIONS)} are)")
+    if activation == "silu":
+        return silu_mul(gate_up)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "act_mul: input must be [tokens, 2 * width]")
+    _dense(gate_up, "act_mul: input")
+    dtype_code(gate_up)
+    out = torch.empty((gate_up.shape[0], gate_up.shape[1] // 2), dtype=gate_up.dtype, device=gate_up.device)
+    backend().act_mul(gate_up, out, ACTIVATIONS[activation])
+    return out
+
+
+# ------------------------------------------------------------------ attention over a cached latent
+def latent_prepare(a: torch.Tensor, q_off: int, q_rank: int, c_off: int, kv_rank: int, rot: int, wq: torch.Tensor,
+                   wc: torch.Tensor | None, eps: float, freqs: torch.Tensor | None, gain: float, positions: torch.Tensor,
+                   slot_mapping: torch.Tensor | None, cache: torch.Tensor | None, out_dtype) -> torch.Tensor:
+    """``a`` [tokens, columns] float32 holds the packed down projections of the step's rows. Returns the query latent
+    (columns q_off ..., RMS-normed with ``wq``) as [tokens, q_rank] in ``out_dtype``; where ``kv_rank`` > 0 and a
+    ``slot_mapping`` is given, stores [RMS-normed columns c_off ... | the ``rot`` columns after them, turned pairwise
+    (2i, 2i + 1) by position * freqs[i], cosine and sine times ``gain``] at the tokens' slots of ``cache``."""
+    T = a.shape[0]
+    _need(a.dim() == 2, "latent_prepare: a must be [tokens, columns]")
+    _dense(a, "latent_prepare: a", dtype=torch.float32)
+    _float32(wq, "latent_prepare: query norm weight", (q_rank,))
+    _dense(positions, "latent_prepare: positions", (T,), torch.int32)
+    _need(out_dtype in _DTYPE_CODE, lambda: f"latent_prepare: rows of {out_dtype}")
+    store = kv_rank > 0 and slot_mapping is not None
+    if store:
+        _float32(wc, "latent_prepare: latent norm weight", (kv_rank,))
+        _dense(slot_mapping, "latent_prepare: slot_mapping", (T,), torch.int32)
+        _need(cache is not None and cache.dim() == 4 and cache.shape[2] == 1 and cache.shape[3] >= kv_rank + rot,
+              lambda: f"latent_prepare: cache of shape {None if cache is None else tuple(cache.shape)} for rows of {kv_rank} + {rot}")
+        _dense(cache, "latent_prepare: cache", dtype=out_dtype)
+        if rot:
+            _dense(freqs, "latent_prepare: frequencies", (rot // 2,), torch.float64)
+    cq = torch.empty((T, q_rank), dtype=out_dtype, device=a.device)
+    backend().latent_prepare(a, q_off, q_rank, c_off, kv_rank if store else 0, rot if store else 0, wq, wc if store else None,
+                             float(eps), freqs if store and rot else None, float(gain), positions,
+                             slot_mapping if store else None, cache if store else None, cq)
+    return cq
+
+
+def head_gemm(x: torch.Tensor, w: torch.Tensor, transposed: bool, N: int, K: int, x_off: int = 0, out: torch.Tensor | None = None,
+              out_off: int = 0, gate: torch.Tensor | None = None, gate_off: int = 0) -> torch.Tensor:
+    """One small matrix per head: out[t, h, out_off : out_off + N] = M_h x[t, h, x_off : x_off + K], sums in float.
+    ``w`` is [heads * K, N] with M_h = w[h K : (h + 1) K]^T (``transposed``: x is multiplied from the left by the
+    block's transpose) or [heads * N, K] with M_h = w[h N : (h + 1) N]. ``gate`` [tokens, columns] float32: the result
+    of (t, h) is multiplied by sigmoid(gate[t, gate_off + h]). ``out``: [tokens, heads, row] to write into."""
+    _need(x.dim() == 3, "head_gemm: x must be [tokens, heads, row]")
+    T, H, x_row = x.shape
+    _dense(x, "head_gemm: x")
+    dtype_code(x)
+    _need(0 <= x_off and x_off + K <= x_row, lambda: f"head_gemm: columns {x_off}+{K} of {x_row}")
+    _dense(w, "head_gemm: w", (H * K, N) if transposed else (H * N, K), x.dtype)
+    if out is None:
+        out = torch.empty((T, H, N), dtype=x.dtype, device=x.device)
+    _need(out.dim() == 3 and tuple(out.shape[:2]) == (T, H) and 0 <= out_off and out_off + N <= out.shape[2],
+          lambda: f"head_gemm: out {tuple(out.shape)} for {N} columns at {out_off}")
+    _dense(out, "head_gemm: out", dtype=x.dtype)
+    if gate is not None:
+        _need(gate.dim() == 2 and gate.shape[0] == T and 0 <= gate_off and gate_off + H <= gate.shape[1],
+              lambda: f"head_gemm: gate {tuple(gate.shape)} for {H} heads at {gate_off}")
+        _dense(gate, "head_gemm: gate", dtype=torch.float32)
+    if transposed:
+        w_head, w_n, w_k = K * N, 1, N
+    else:
+        w_head, w_n, w_k = N * K, K, 1
+    backend().head_gemm(x, x_off, x_row, w, w_head, w_n, w_k, out, out_off, out.shape[2], gate, gate_off, N, K)
+    return out
+
+
+def rotate_interleaved(src: torch.Tensor, s_off: int, dst: torch.Tensor, d_off: int, rot: int, freqs: torch.Tensor,
+                       gain: float, positions: torch.Tensor) -> torch.Tensor:
+    """dst[t, h, d_off + j] = src[t, h, s_off + j] turned, j < rot: pairs (2i, 2i + 1) by position * freqs[i]."""
+    _need(src.dim() == 3 and dst.dim() == 3 and tuple(src.shape[:2]) == tuple(dst.shape[:2]),
+          "rotate_interleaved: src and dst must be [tokens, heads, row]")
+    _dense(src, "rotate_interleaved: src")
+    _dense(dst, "rotate_interleaved: dst", dtype=src.dtype)
+    dtype_code(src)
+    _need(rot > 0 and rot % 2 == 0 and 0 <= s_off and s_off + rot <= src.shape[2] and 0 <= d_off and d_off + rot <= dst.shape[2],
+          lambda: f"rotate_interleaved: {rot} entries at {s_off} of {src.shape[2]} into {d_off} of {dst.shape[2]}")
+    _dense(freqs, "rotate_interleaved: frequencies", (rot // 2,), torch.float64)
+    _dense(positions, "rotate_interleaved: positions", (src.shape[0],), torch.int32)
+    backend().rotate_interleaved(src, s_off, dst, d_off, rot, freqs, float(gain), positions)
+    return dst
+
+
+# ------------------------------------------------------------------ a feed-forward of many small experts
+def route_topk(h: torch.Tensor, router: torch.Tensor, top: int):
+    """(numbers [tokens, top] int32, scores [tokens, top] float32) of the ``top`` experts with the largest
+    sigmoid(router . h), logits summed in float; the largest first, the lower number among equals."""
+    _need(h.dim() == 2, "route_topk: h must be [tokens, width]")
+    _dense(h, "route_topk: h")
+    dtype_code(h)
+    _need(router.dim() == 2, "route_topk: the router must be [experts, width]")
+    _float32(router, "route_topk: router", (router.shape[0], h.shape[1]))
+    _need(0 < top <= router.shape[0], lambda: f"route_topk: {top} of {router.shape[0]} experts")
+    ids = torch.empty((h.shape[0], top), dtype=torch.int32, device=h.device)
+    scores = torch.empty((h.shape[0], top), dtype=torch.float32, device=h.device)
+    backend().route_topk(h, router, ids, scores)
+    return ids, scores
+
+
+def routed_experts(h: torch.Tensor, ids: torch.Tensor, scores: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
+                   activation: str = "silu") -> torch.Tensor:
+    """sum over a token's experts e (``ids``) of D_e (act(G_e x) * (U_e x)), x = score * h: the score multiplies the
+    expert's input. ``gate_up`` [experts, 2 ff, width] (gate rows, then up rows), ``down`` [experts, width, ff]."""
+    _need(h.dim() == 2, "routed_experts: h must be [tokens, width]")
+    T, W = h.shape
+    _dense(h, "routed_experts: h")
+    dtype_code(h)
+    _need(activation in ACTIVATIONS, lambda: f"routed_experts: activation {activation!r}")
+    _need(gate_up.dim() == 3 and gate_up.shape[2] == W and gate_up.shape[1] % 2 == 0, "routed_experts: gate_up must be [experts, 2 ff, width]")
+    E, F = gate_up.shape[0], gate_up.shape[1] // 2
+    _dense(gate_up, "routed_experts: gate_up", dtype=h.dtype)
+    _dense(down, "routed_experts: down", (E, W, F), h.dtype)
+    _need(ids.dim() == 2 and ids.shape[0] == T, "routed_experts: ids must be [tokens, top]")
+    _dense(ids, "routed_experts: ids", dtype=torch.int32)
+    _dense(scores, "routed_experts: scores", tuple(ids.shape), torch.float32)
+    u = torch.empty((T * ids.shape[1], F), dtype=h.dtype, device=h.device)
+    backend().experts_gate_up(h, ids, scores, gate_up, u, ACTIVATIONS[activation])
+    out = torch.empty((T, W), dtype=h.dtype, device=h.device)
+    backend().experts_down(u, ids, down, out)
+    return out
 
 # ------------------------------------------------------------------ layers that are not the pre-norm kind
 def _float32(t: torch.Tensor, name: str, shape: tuple) -> None:

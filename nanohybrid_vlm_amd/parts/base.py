@@ -35,10 +35,18 @@ class PagedKVNeed:
     window: int | None = None     # None: all keys; n: only the last n are read
     value_dim: int | None = None  # size of a value head where it is not ``head_dim``
     chunk: int | None = None      # n: a query reads only the keys of its own block of n positions (counted from 0)
+    # True: what a token stores is one row per head that serves as its key and, whole, as its value (a latent that
+    # keys and values are made of): there is no value tensor, readers get the key tensor for both
+    values_in_keys: bool = False
 
     @property
     def value_size(self) -> int:
         return self.head_dim if self.value_dim is None else self.value_dim
+
+    @property
+    def stored_per_head(self) -> int:
+        """Entries that a token stores per head."""
+        return self.head_dim if self.values_in_keys else self.head_dim + self.value_size
 
 
 @dataclass(frozen=True)
@@ -157,3 +165,4 @@ FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block")
+EMBEDDINGS = Registry("embedding")

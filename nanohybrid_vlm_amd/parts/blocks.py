@@ -121,3 +121,54 @@ class ParallelDepthMixBlock(Part):
             step.scratch["normed_ahead"] = (next_norm, out, normed)
             return out, None
         return ops.depth_mix(hidden, mixed, fed, results, self.depth_index, self.depth_weight), None
+
+
+@BLOCKS.register("parallel_two_norms")
+class ParallelTwoNormsBlock(Part):
+    """x <- x + (mixer(norm_a(x)) + feed_forward(norm_b(x))): both norms read the same x. The stream x is float32 and is
+    what the block takes and returns as ``hidden`` (no residual beside it). The two norms share their mean and
+    variance, so one kernel makes both; the additions of a block are left to the kernel that norms for the block after
+    it (``pending`` in ``step.scratch``), or made by a kernel of their own after the last block. The feed-forward may
+    be absent (then there is no second norm)."""
+
+    norm_slots = ("mixer_norm", "feed_forward_norm")
+    norms_ahead = True            # the model tells the block whether a block follows (``next_norm`` is that block's ``norm``)
+
+    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+        if feed_forward is not None and feed_forward_norm.eps != mixer_norm.eps:
+            raise ValueError("the two norms of this block share their statistics and so their eps")
+        self.row_dtype = None
+
+    @property
+    def norm(self):
+        """What the block before this one is shown as the norm that takes its result: this block adds what is
+        pending itself, in its norms' kernel."""
+        return self
+
+    def children(self):
+        out = {"mixer_norm": self.mixer_norm, "mixer": self.mixer}
+        if self.feed_forward is not None:
+            out["feed_forward_norm"] = self.feed_forward_norm
+            out["feed_forward"] = self.feed_forward
+        return out
+
+    def forward(self, hidden, residual, step, cache, next_norm=None):
+        if residual is not None:
+            raise ValueError("this block carries its stream itself and takes no residual beside it")
+        if hidden.dtype != torch.float32:
+            hidden = hidden.float()
+        pending = step.scratch.pop("pending_additions", None)
+        add = pending[1] if pending is not None and pending[0] is hidden else ()
+        dtype = self.row_dtype or torch.float32
+        a, b = self.mixer_norm, self.feed_forward_norm
+        second = (b.weight, b.bias) if self.feed_forward is not None else None
+        h1, h2 = ops.layernorm_pair(hidden, (a.weight, a.bias), second, a.eps, dtype, add=add)
+        mixed = self.mixer.forward(h1, step, cache)
+        fed = self.feed_forward.forward(h2, step) if self.feed_forward is not None else None
+        if isinstance(next_norm, ParallelTwoNormsBlock):
+            step.scratch["pending_additions"] = (hidden, (mixed, fed))
+        else:
+            ops.add_streams_(hidden, mixed, fed)
+        return hidden, None

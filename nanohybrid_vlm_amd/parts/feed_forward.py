@@ -13,9 +13,13 @@ class SwiGLU(Part):
     ``intermediate_size`` rows are the gate (nanovllm/layers/linear.py:102-108,
     nanovllm/layers/activation.py:10-11)."""
 
-    def __init__(self, hidden_size: int, intermediate_size: int):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
+        """``activation``: what the gate passes, "silu" (the reference's) or "gelu_tanh"."""
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not known ({sorted(ops.ACTIVATIONS)} are)")
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
+        self.activation = activation
         self.gate_up_weight = None
         self.down_weight = None
 
@@ -33,4 +37,39 @@ class SwiGLU(Part):
         return self.gate_up_weight, True
 
     def forward(self, x, step, add_to=None):
+        if self.activation != "silu":
+            return ops.linear(ops.act_mul(ops.linear(x, self.gate_up_weight), self.activation), self.down_weight, add_to=add_to)
         return ops.linear(ops.gated_linear(x, self.gate_up_weight), self.down_weight, add_to=add_to)
+
+
+@FEED_FORWARDS.register("routed_experts")
+class RoutedExperts(Part):
+    """``num_experts`` gated feed-forwards of inner size ``expert_size`` without biases, of which every token uses the
+    ``top`` with the largest score s_e = sigmoid(router_e . x) (logits in float32). The scores are taken as they are
+    (not renormalised) and multiply the experts' inputs: y = sum over chosen e of D_e (act(G_e s_e x) * (U_e s_e x)).
+    All experts' matrices lie in two tensors, [experts * 2 expert_size, width] (per expert its gate rows, then its
+    up rows) and [experts * width, expert_size]."""
+
+    def __init__(self, hidden_size: int, num_experts: int, top: int, expert_size: int, activation: str = "silu"):
+        if not 0 < top <= num_experts or min(hidden_size, expert_size) <= 0:
+            raise ValueError(f"{top} of {num_experts} experts of size {expert_size}")
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not known ({sorted(ops.ACTIVATIONS)} are)")
+        self.hidden_size, self.num_experts, self.top, self.expert_size = hidden_size, num_experts, top, expert_size
+        self.activation = activation
+
+    def param_specs(self):
+        E, F, W = self.num_experts, self.expert_size, self.hidden_size
+        return {"router.weight": ParamSpec((E, W), always_float32=True),
+                "gate_up.weight": ParamSpec((E * 2 * F, W)),
+                "down.weight": ParamSpec((E * W, F))}
+
+    def bind(self, params):
+        E, F, W = self.num_experts, self.expert_size, self.hidden_size
+        self.router_weight = params["router.weight"]
+        self.gate_up_weight = params["gate_up.weight"].view(E, 2 * F, W)
+        self.down_weight = params["down.weight"].view(E, W, F)
+
+    def forward(self, x, step):
+        ids, scores = ops.route_topk(x, self.router_weight, self.top)
+        return ops.routed_experts(x, ids, scores, self.gate_up_weight, self.down_weight, self.activation)

@@ -14,7 +14,7 @@ import torch
 from ..native import ops
 from dataclasses import replace
 
-from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheView, CombinedNeed, PagedKVNeed, ParamSpec,
+from .base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheView, CombinedNeed, PagedKVNeed, ParamSpec,
                    Part, StateNeed)
 
 
@@ -65,6 +65,7 @@ class ModelSpec:
     logit_cap: float | None = None            # logits become cap * tanh(logits / cap)
     position_axes: int = 1                    # coordinates of a token's position (a step carries [axes, tokens])
     embed_norm: dict | None = None            # a norm that the embedding's rows pass before the first layer
+    embedding: dict | None = None             # None: the rows of the table; else a registered embedding that uses the table
 
     def order(self) -> list[RunEntry]:
         if self.run_order is None:
@@ -101,6 +102,8 @@ class DecoderModel(Part):
             self.layers.append(BLOCKS.build(ls.block, offered=options, mixer=mixer, feed_forward=ff, **norms))
         self.final_norm = NORMS.build(spec.final_norm, offered=options)
         self.embed_norm = NORMS.build(spec.embed_norm, offered=options) if spec.embed_norm is not None else None
+        self.embedding = EMBEDDINGS.build(spec.embedding, offered=options) if spec.embedding is not None else None
+        self.embedding_state = None
         self.run_order = spec.order()
         for i, e in enumerate(self.run_order):
             if not 0 <= e.layer < len(self.layers):
@@ -134,6 +137,8 @@ class DecoderModel(Part):
         out["final_norm"] = self.final_norm
         if self.embed_norm is not None:
             out["embed_norm"] = self.embed_norm
+        if self.embedding is not None:
+            out["embedding"] = self.embedding
         return out
 
     def bind(self, params):
@@ -171,6 +176,15 @@ class DecoderModel(Part):
                     out[e.cache] = replace(lent, chunk=None)
         return out
 
+    def embedding_state_need(self) -> StateNeed | None:
+        """What the embedding keeps per request (beside the run-order entries' caches), if anything."""
+        need = getattr(self.embedding, "state_need", None)
+        return need() if need is not None else None
+
+    def attach_embedding_state(self, pool: dict | None) -> None:
+        """``pool``: name -> [slots, ...] for what ``embedding_state_need`` names."""
+        self.embedding_state = pool
+
     def attach_cache(self, views: list[CacheView]) -> None:
         """``views[i]`` is the cache of run-order entry i (for a borrowing entry: the lender's, with writes off)."""
         if len(views) != len(self.run_order):
@@ -180,7 +194,10 @@ class DecoderModel(Part):
     # -- the forward pass -------------------------------------------------
     def forward(self, step) -> torch.Tensor:
         """Hidden states after the final norm, for the rows whose logits are wanted only: [n, hidden]."""
-        hidden = ops.embed(step.input_ids, self.embed_weight, self.spec.embed_scale)
+        if self.embedding is not None:
+            hidden = self.embedding.forward(step, self.embed_weight, self.embedding_state)
+        else:
+            hidden = ops.embed(step.input_ids, self.embed_weight, self.spec.embed_scale)
         if self.embed_norm is not None:
             hidden = self.embed_norm.forward(hidden)
         residual = None

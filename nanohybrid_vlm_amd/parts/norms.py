@@ -77,3 +77,26 @@ class ScalarRMSNorm(Part):
         if out_dtype is None:
             out_dtype = {"same": x.dtype, "float32": torch.float32, "rows": self.row_dtype or x.dtype}[self.output]
         return ops.scalar_rmsnorm(x, self.weight, self.eps, out_dtype=out_dtype)
+
+
+@NORMS.register("layernorm")
+class LayerNorm(Part):
+    """y = (x - mean) / sqrt(variance + eps) * weight + bias over the width, the variance being the mean of the squared
+    deviations. It reads a float32 stream and gives rows of the model's element type; statistics, weight and bias
+    are float32. Two such norms of one stream share their statistics: ``ops.layernorm_pair`` takes both at once (see
+    the block ``parallel_two_norms``)."""
+
+    def __init__(self, size: int, eps: float):
+        self.size, self.eps = size, eps
+        self.weight = self.bias = None
+        self.row_dtype = None         # set when the model's weights are bound
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.size,), init="norm", always_float32=True),
+                "bias": ParamSpec((self.size,), init="zeros", always_float32=True)}
+
+    def forward(self, x, out_dtype=None) -> torch.Tensor:
+        if x.dtype != torch.float32:
+            x = x.float()
+        y, _ = ops.layernorm_pair(x, (self.weight, self.bias), None, self.eps, out_dtype or self.row_dtype or torch.float32)
+        return y

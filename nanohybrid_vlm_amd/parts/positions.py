@@ -107,3 +107,48 @@ class RotaryFrequencies(PositionEncoding):
         self.freqs = self.freqs.to(device)
         self._others = {n: f.to(device) for n, f in self._others.items()}
         return self
+
+
+@POSITION_ENCODINGS.register("yarn_frequencies")
+class YarnFrequencies(PositionEncoding):
+    """Rotation given by frequencies that are scaled part by part (YaRN): with f_i = base^(-2 i / rotary_dim) and
+        dim(t) = rotary_dim ln(original / (2 pi t)) / (2 ln base),  lo = max(floor(dim(fast)), 0),
+        hi = min(ceil(dim(slow)), rotary_dim - 1),  ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1),
+    pair i turns by position * (f_i / factor * ramp_i + f_i (1 - ramp_i)), and cosines and sines are multiplied by
+    ``gain()`` = 0.1 ln(factor) + 1. Without ``factor`` the frequencies are the plain ones and the gain is 1. The
+    frequencies are kept in float64: the kernels take the angle in double before they take its sine and cosine."""
+
+    def __init__(self, rotary_dim: int, base: float, max_position: int, factor: float | None = None,
+                 original: float | None = None, fast: float | None = None, slow: float | None = None, device=None):
+        if rotary_dim % 2 or rotary_dim < 0:
+            raise ValueError(f"rotary_dim must be even and not negative, got {rotary_dim}")
+        self.rotary_dim, self.base, self.max_position = rotary_dim, float(base), max_position
+        self.factor = None if factor is None else float(factor)
+        i = torch.arange(rotary_dim // 2, dtype=torch.float64)
+        f = self.base ** (-2.0 * i / max(rotary_dim, 1))
+        self._gain = 1.0
+        if self.factor is not None:
+            if not self.factor > 0 or None in (original, fast, slow):
+                raise ValueError("scaled frequencies need a positive factor, and original, fast and slow")
+            import math
+
+            def dim_of(turns: float) -> float:
+                return rotary_dim * math.log(original / (2 * math.pi * turns)) / (2 * math.log(self.base))
+
+            lo = max(math.floor(dim_of(fast)), 0)
+            hi = min(math.ceil(dim_of(slow)), rotary_dim - 1)
+            ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+            f = f / self.factor * ramp + f * (1 - ramp)
+            self._gain = 0.1 * math.log(self.factor) + 1.0
+        self.freqs = f if device is None else f.to(device)
+
+    def frequencies(self) -> torch.Tensor:
+        """[rotary_dim / 2] float64."""
+        return self.freqs
+
+    def gain(self) -> float:
+        return self._gain
+
+    def to(self, device):
+        self.freqs = self.freqs.to(device)
+        return self

@@ -127,6 +127,113 @@ class EmulatedBackend:
         if gain is not None:
             normed.copy_((total * (gain / torch.sqrt(total.pow(2).mean(-1, keepdim=True) + eps))).to(normed.dtype))
 
+    # -- two norms side by side, a hashed pair embedding
+    def embed_pair_hash(self, ids, table, pair_table, out, batch, state_slots, prev_state, buckets, mul_prev, mul_cur):
+        cu = batch.cu_seqlens_q.tolist()
+        for r in range(batch.num_requests):
+            lo, hi = cu[r], cu[r + 1]
+            if hi <= lo:
+                continue
+            slot = int(state_slots[r])
+            prev = int(prev_state[slot])
+            for t in range(lo, hi):
+                tok = int(ids[t])
+                row = buckets if int(batch.positions[t]) == 0 else (prev * mul_prev + tok * mul_cur) % buckets
+                out[t] = table[tok].float() + pair_table[row].float()
+                prev = tok
+            prev_state[slot] = prev
+
+    def layernorm_pair(self, x, a, b, w1, b1, y1, w2, b2, y2, eps, rows_dtype):
+        s = x
+        if a is not None:
+            s = s + a.float()
+        if b is not None:
+            s = s + b.float()
+        if a is not None or b is not None:
+            x.copy_(s)
+        mean = s.mean(-1, keepdim=True)
+        n = (s - mean) / torch.sqrt(((s - mean) ** 2).mean(-1, keepdim=True) + eps)
+        if y1 is not None:
+            y1.copy_((n * w1 + b1).to(y1.dtype))
+        if y2 is not None:
+            y2.copy_((n * w2 + b2).to(y2.dtype))
+
+    def add_streams(self, x, a, b):
+        x.add_(a.float() if b is None else a.float() + b.float())
+
+    @staticmethod
+    def _act(z, act):
+        if act == 1:
+            return 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        return z * torch.sigmoid(z)
+
+    def act_mul(self, gu, out, act):
+        I = out.shape[1]
+        out.copy_((self._act(gu[:, :I].float(), act) * gu[:, I:].float()).to(out.dtype))
+
+    # -- attention over a cached latent
+    @staticmethod
+    def _turn_pairs(t, positions, freqs, gain):
+        ang = positions.double()[:, None] * freqs[None, :]
+        cos, sin = (ang.cos() * gain).float(), (ang.sin() * gain).float()
+        while cos.dim() < t.dim():
+            cos, sin = cos.unsqueeze(1), sin.unsqueeze(1)
+        u, v = t[..., 0::2], t[..., 1::2]
+        out = torch.empty_like(t)
+        out[..., 0::2] = u * cos - v * sin
+        out[..., 1::2] = v * cos + u * sin
+        return out
+
+    def latent_prepare(self, a, q_off, q_rank, c_off, kv_rank, rot, wq, wc, eps, freqs, gain, positions, slot_mapping,
+                       cache, cq):
+        q = a[:, q_off:q_off + q_rank]
+        cq.copy_((q / torch.sqrt(q.pow(2).mean(-1, keepdim=True) + eps) * wq).to(cq.dtype))
+        if kv_rank == 0 or slot_mapping is None:
+            return
+        c = a[:, c_off:c_off + kv_rank]
+        rows = [c / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + eps) * wc]
+        if rot:
+            rows.append(self._turn_pairs(a[:, c_off + kv_rank:c_off + kv_rank + rot], positions, freqs, gain))
+        rows = torch.cat(rows, dim=-1).to(cache.dtype)
+        ok = slot_mapping >= 0
+        cache.view(-1, cache.shape[-1])[slot_mapping[ok].long(), :kv_rank + rot] = rows[ok]
+
+    def head_gemm(self, x, x_off, x_row, w, w_head, w_n, w_k, y, y_off, y_row, gate, gate_off, N, K):
+        T, H = x.shape[0], x.shape[1]
+        m = torch.as_strided(w, (H, N, K), (w_head, w_n, w_k)).float()
+        r = torch.einsum("thk,hnk->thn", x[:, :, x_off:x_off + K].float(), m)
+        if gate is not None:
+            r = r * torch.sigmoid(gate[:, gate_off:gate_off + H])[:, :, None]
+        y[:, :, y_off:y_off + N] = r.to(y.dtype)
+
+    def rotate_interleaved(self, src, s_off, dst, d_off, rot, freqs, gain, positions):
+        dst[:, :, d_off:d_off + rot] = self._turn_pairs(src[:, :, s_off:s_off + rot].float(), positions, freqs, gain).to(dst.dtype)
+
+    # -- a feed-forward of many small experts
+    def route_topk(self, h, router, ids, scores):
+        z = h.float() @ router.T
+        top = ids.shape[1]
+        order = torch.sort(z, dim=-1, descending=True, stable=True).indices[:, :top]
+        ids.copy_(order.to(torch.int32))
+        scores.copy_(torch.sigmoid(torch.gather(z, 1, order)))
+
+    def experts_gate_up(self, h, ids, scores, gate_up, u, act):
+        T, top = ids.shape
+        F = gate_up.shape[1] // 2
+        for t in range(T):
+            for j in range(top):
+                e, s = int(ids[t, j]), scores[t, j]
+                gu = gate_up[e].float() @ h[t].float()
+                u[t * top + j] = (self._act(s * gu[:F], act) * (s * gu[F:])).to(u.dtype)
+
+    def experts_down(self, u, ids, down, out):
+        T, top = ids.shape
+        for t in range(T):
+            total = torch.zeros(out.shape[1])
+            for j in range(top):
+                total = total + down[int(ids[t, j])].float() @ u[t * top + j].float()
+            out[t] = total.to(out.dtype)
+
     @staticmethod
     def _turned(t, positions, freqs, sign=1.0):
         half = freqs.shape[0]
