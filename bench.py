@@ -19,7 +19,7 @@ For these two ``value`` is generated tokens a second over the whole run, prompts
 ``--workload projections`` is a diagnosis, not the benchmark: a layer's matrix products alone, cold, beside a kernel
 that only reads the same bytes (see ``bench_projections``).
 
-``--workload design --shape pevazen-1b|pevazen-8b [--layers L]``: a model of the Pevazen design (attention and
+``--workload design --shape pevazen-1b|pevazen-8b|fazovik-1b|fazovik-8b [--layers L]``: a model of the Pevazen or the Fazovik design (attention and
 recurrent layers side by side, see ``architectures/pevazen.py``) beside a Qwen3 model of the same width, heads,
 feed-forward size, vocabulary and number of layers: one prompt of ``--prompt-tokens`` in one step, decoding at
 ``--batch`` requests, and the time of every own kernel in one eager step of each kind (see ``bench_design``).
@@ -422,17 +422,25 @@ def bench_design(args):
     from nanohybrid_vlm_amd.engine.runner import StepEntry
     from nanohybrid_vlm_amd.native import ops
 
-    name = args.shape if args.shape.startswith("pevazen") else "pevazen-1b"
+    name = args.shape if args.shape.startswith(("pevazen", "fazovik")) else "pevazen-1b"
+    design = name.split("-")[0]
     new = json.loads(json.dumps(named_shapes()[name]))
     layers = args.layers or min(8, len(new["layers"]))
     new["layers"] = new["layers"][:layers]
-    a = new["layers"][1]["mixer"]
-    twin = qwen3_shape(layers, new["width"], a["heads"], a["kv_heads"], a["dim"], new["layers"][0]["mlp"]["ff"], vocab=new["vocab"])
+    if design == "fazovik":
+        # the twin has as many heads, of the size of this design's value heads, a quarter as many key/value heads, and
+        # the dense layers' inner size in every layer
+        a = new["layers"][0]["mixer"]
+        twin = qwen3_shape(layers, new["width"], a["heads"], max(1, a["heads"] // 4), a["vdim"], new["layers"][0]["mlp"]["ff"],
+                           vocab=new["vocab"])
+    else:
+        a = new["layers"][1]["mixer"]
+        twin = qwen3_shape(layers, new["width"], a["heads"], a["kv_heads"], a["dim"], new["layers"][0]["mlp"]["ff"], vocab=new["vocab"])
     batch, T = args.batch or 8, args.prompt_tokens or 2048
     context = args.context or (T + 512)
     pages = (batch + 1) * -(-context // args.block_size) + 1
     out = {}
-    for label, raw in (("pevazen", new), ("qwen3", twin)):
+    for label, raw in ((design, new), ("qwen3", twin)):
         llm = LLM(raw, random_weights=0, dtype=args.dtype, kvcache_block_size=args.block_size, max_num_seqs=max(batch, 1),
                   enforce_eager=args.eager, num_kvcache_blocks=pages, max_num_batched_tokens=max(args.token_budget, T, batch),
                   max_model_len=context, scheduler_policy="prefill_first")
@@ -479,13 +487,13 @@ def bench_design(args):
         llm.exit()
         del llm, runner
         torch.cuda.empty_cache()
-    line = {"metric": f"Pevazen ({name}, {layers} layers) beside Qwen3 of equal sizes: prefill of {T} tokens and decode at batch {batch}",
-            "value": out["pevazen"]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-            "ms_per_step": out["pevazen"]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+    line = {"metric": f"{design.capitalize()} ({name}, {layers} layers) beside Qwen3 of equal sizes: prefill of {T} tokens and decode at batch {batch}",
+            "value": out[design]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": out[design]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random token ids, random weights",
             "config": {"model": name, "layers": layers, "width": new["width"], "global_batch": batch, "prompt_len": T,
                        "seq_len": context, "parallelism": "single GPU", "graphs": not args.eager},
-            "pevazen": out["pevazen"], "qwen3": out["qwen3"]}
+            design: out[design], "qwen3": out["qwen3"]}
     print(json.dumps(line), flush=True)
     return 0
 
