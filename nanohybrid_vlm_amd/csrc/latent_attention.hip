@@ -4,6 +4,7 @@
 //                           [RMS-normed c | rotated r] stored at the step's slots
 //   nhv_head_gemm           y[t, h, :] = M_h x[t, h, :] for a matrix per head (strides say which way M_h lies), with an
 //                           optional sigmoid gate per (token, head) on the result
+//   nhv_head_gemm_fewrows   the same for up to 16 rows, with the turning of the queries' rotated part in the same launch
 //   nhv_rotate_interleaved  the rotated part of every query head, turned by position and copied beside the rest
 // Pairs (2i, 2i + 1) turn by angle = position * freqs[i]; cosine and sine are multiplied by ``gain``. The frequencies
 // come as doubles and the product with the position is taken and brought into [-pi, pi] in double (a float product
@@ -158,6 +159,84 @@ extern "C" int nhv_head_gemm(const void* x, long long xs_t, long long xs_h, cons
   else
     return nhv_fail("head_gemm: unknown dtype %d", dtype);
   NHV_LAUNCH_CHECK("head_gemm");
+  return 0;
+}
+
+// The same for up to 16 rows (a decoding step): a block owns 256 outputs of one head, keeps the head's rows of x in LDS
+// as floats and gives every thread one output of all rows; k rises as above, so the sums are the same bits. One more
+// block a head may turn the rotated part of x and copy it beside the outputs (``rot`` entries from x_rot_off to
+// y_rot_off), which saves the launch of nhv_rotate_interleaved.
+template <typename T>
+__global__ __launch_bounds__(256) void head_gemm_fewrows_kernel(const T* __restrict__ x, long long xs_t, long long xs_h,
+                                                                const T* __restrict__ w, long long ws_h, long long ws_n,
+                                                                long long ws_k, T* __restrict__ y, long long ys_t,
+                                                                long long ys_h, const float* __restrict__ gate,
+                                                                long long gs_t, int rows, int N, int K, int n_chunks, int rot,
+                                                                int x_rot_off, int y_rot_off, const double* __restrict__ freqs,
+                                                                float gain, const int* __restrict__ positions) {
+  extern __shared__ float xs[];              // 16 x K
+  const int h = blockIdx.y;
+  if ((int)blockIdx.x == n_chunks) {         // the rotated part
+    for (int i = threadIdx.x; i < rows * (rot / 2); i += blockDim.x) {
+      const int t = i / (rot / 2), p = i % (rot / 2);
+      float sn, cs;
+      nhv_turn_angle(positions[t], freqs[p], gain, &sn, &cs);
+      const T* s = x + (size_t)t * xs_t + (size_t)h * xs_h + x_rot_off + 2 * p;
+      T* d = y + (size_t)t * ys_t + (size_t)h * ys_h + y_rot_off + 2 * p;
+      const float u = to_f32(s[0]), v = to_f32(s[1]);
+      d[0] = from_f32<T>(u * cs - v * sn);
+      d[1] = from_f32<T>(v * cs + u * sn);
+    }
+    return;
+  }
+  for (int i = threadIdx.x; i < 16 * K; i += blockDim.x) {
+    const int t = i / K, k = i % K;
+    xs[i] = t < rows ? to_f32(x[(size_t)t * xs_t + (size_t)h * xs_h + k]) : 0.f;
+  }
+  __syncthreads();
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= N) return;
+  float acc[16];
+#pragma unroll
+  for (int t = 0; t < 16; ++t) acc[t] = 0.f;
+  const T* wn = w + (size_t)h * ws_h + (size_t)n * ws_n;
+  for (int k = 0; k < K; ++k) {
+    const float wv = to_f32(wn[(size_t)k * ws_k]);
+#pragma unroll
+    for (int t = 0; t < 16; ++t) acc[t] = fmaf(xs[t * K + k], wv, acc[t]);
+  }
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    if (t >= rows) break;
+    float v = acc[t];
+    if (gate != nullptr) v *= 1.0f / (1.0f + expf(-gate[(size_t)t * gs_t + h]));
+    y[(size_t)t * ys_t + (size_t)h * ys_h + n] = from_f32<T>(v);
+  }
+}
+
+extern "C" int nhv_head_gemm_fewrows(const void* x, long long xs_t, long long xs_h, const void* w, long long ws_h,
+                                     long long ws_n, long long ws_k, void* y, long long ys_t, long long ys_h, const void* gate,
+                                     long long gs_t, int rows, int H, int N, int K, int rot, int x_rot_off, int y_rot_off,
+                                     const void* freqs, float gain, const void* positions, int dtype, void* stream) {
+  NHV_REQUIRE(rows > 0 && rows <= 16 && H > 0 && H <= 65535 && N > 0 && K > 0 && K <= 1024,
+              "head_gemm_fewrows: bad sizes rows=%d (up to 16) H=%d N=%d K=%d (up to 1024)", rows, H, N, K);
+  NHV_REQUIRE(rot >= 0 && rot % 2 == 0 && (rot == 0 || (freqs != nullptr && positions != nullptr)),
+              "head_gemm_fewrows: a rotated part of %d entries needs frequencies and positions", rot);
+  const int n_chunks = (N + 255) / 256;
+  const dim3 grid(n_chunks + (rot > 0 ? 1 : 0), H);
+  const size_t lds = 16 * (size_t)K * sizeof(float);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == NHV_F32)
+    hipLaunchKernelGGL(head_gemm_fewrows_kernel<float>, grid, dim3(256), lds, s, (const float*)x, xs_t, xs_h, (const float*)w,
+                       ws_h, ws_n, ws_k, (float*)y, ys_t, ys_h, (const float*)gate, gs_t, rows, N, K, n_chunks, rot, x_rot_off,
+                       y_rot_off, (const double*)freqs, gain, (const int*)positions);
+  else if (dtype == NHV_BF16)
+    hipLaunchKernelGGL(head_gemm_fewrows_kernel<bf16_t>, grid, dim3(256), lds, s, (const bf16_t*)x, xs_t, xs_h,
+                       (const bf16_t*)w, ws_h, ws_n, ws_k, (bf16_t*)y, ys_t, ys_h, (const float*)gate, gs_t, rows, N, K,
+                       n_chunks, rot, x_rot_off, y_rot_off, (const double*)freqs, gain, (const int*)positions);
+  else
+    return nhv_fail("head_gemm_fewrows: unknown dtype %d", dtype);
+  NHV_LAUNCH_CHECK("head_gemm_fewrows");
   return 0;
 }
 

@@ -1,6 +1,5 @@
 // A feed-forward made of many small gated feed-forwards of which every token uses a few.
-//   nhv_route_topk        float router logits of a row, a score per expert (sigmoid), the ``top`` largest: their numbers
-//                         and scores
+//   nhv_route_topk        from a row's float router logits the ``top`` largest: their numbers and scores (sigmoid)
 //   nhv_experts_gate_up   for every (token, chosen expert): act(s G_e h) * (s U_e h), s the score: the expert's input is
 //                         s h, and a product is linear in its rows, so the score multiplies the finished float sums
 //   nhv_experts_down      out[t] = sum over the token's experts of D_e u[t, j]
@@ -10,24 +9,16 @@
 #include "nhv_common.h"
 #include <math.h>
 
-template <typename T>
-__global__ __launch_bounds__(256) void route_topk_kernel(const T* __restrict__ h, const float* __restrict__ router,
-                                                         int* __restrict__ ids, float* __restrict__ scores, int W, int E,
-                                                         int top) {
-  extern __shared__ float z[];               // E logits
-  const int t = blockIdx.x;
+// z [T, E] float logits. One wave per token: the ``top`` largest in turn, the lower number among equals.
+__global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict__ logits, int* __restrict__ ids,
+                                                         float* __restrict__ scores, int T, int E, int top) {
+  extern __shared__ float z_all[];           // 4 waves x E logits
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const T* x = h + (size_t)t * W;
-  for (int e = wave; e < E; e += 4) {
-    const float* w = router + (size_t)e * W;
-    float s = 0.f;
-    for (int k = lane; k < W; k += NHV_WAVE) s = fmaf(w[k], to_f32(x[k]), s);
-    s = wave_sum(s);
-    if (lane == 0) z[e] = s;
-  }
-  __syncthreads();
-  if (wave != 0) return;
-  // the largest first; among equal logits the lower number. A chosen expert's logit becomes -inf.
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= T) return;
+  float* z = z_all + (size_t)wave * E;
+  for (int e = lane; e < E; e += NHV_WAVE) z[e] = logits[(size_t)t * E + e];
+  __builtin_amdgcn_wave_barrier();
   for (int j = 0; j < top; ++j) {
     float best = -INFINITY;
     int at = 0x7fffffff;
@@ -41,29 +32,20 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const T* __restrict__ h
       const int oa = __shfl_xor(at, o, NHV_WAVE);
       if (ov > best || (ov == best && oa < at)) { best = ov; at = oa; }
     }
+    if (at == 0x7fffffff) at = 0;            // (every logit is no number: the first expert)
     if (lane == 0) {
       ids[(size_t)t * top + j] = at;
       scores[(size_t)t * top + j] = 1.0f / (1.0f + expf(-best));
-      z[at] = -INFINITY;
+      z[at] = -INFINITY;                     // a chosen expert is out of the next rounds
     }
     __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
   }
 }
 
-extern "C" int nhv_route_topk(const void* h, const void* router, void* ids, void* scores, int T, int W, int E, int top,
-                              int dtype, void* stream) {
-  NHV_REQUIRE(T > 0 && W > 0 && E > 0 && top > 0 && top <= E && E <= 8192, "route_topk: bad sizes T=%d W=%d E=%d top=%d", T, W, E, top);
-  hipStream_t s = (hipStream_t)stream;
-  const size_t lds = (size_t)E * sizeof(float);
-  if (dtype == NHV_F32)
-    hipLaunchKernelGGL(route_topk_kernel<float>, dim3(T), dim3(256), lds, s, (const float*)h, (const float*)router,
-                       (int*)ids, (float*)scores, W, E, top);
-  else if (dtype == NHV_BF16)
-    hipLaunchKernelGGL(route_topk_kernel<bf16_t>, dim3(T), dim3(256), lds, s, (const bf16_t*)h, (const float*)router,
-                       (int*)ids, (float*)scores, W, E, top);
-  else
-    return nhv_fail("route_topk: unknown dtype %d", dtype);
+extern "C" int nhv_route_topk(const void* logits, void* ids, void* scores, int T, int E, int top, void* stream) {
+  NHV_REQUIRE(T > 0 && E > 0 && top > 0 && top <= E && E <= 8192, "route_topk: bad sizes T=%d E=%d top=%d", T, E, top);
+  hipLaunchKernelGGL(route_topk_kernel, dim3((T + 3) / 4), dim3(256), 4 * (size_t)E * sizeof(float), (hipStream_t)stream,
+                     (const float*)logits, (int*)ids, (float*)scores, T, E, top);
   NHV_LAUNCH_CHECK("route_topk");
   return 0;
 }
@@ -71,6 +53,25 @@ extern "C" int nhv_route_topk(const void* h, const void* router, void* ids, void
 __device__ __forceinline__ float nhv_expert_act(float z, int act) {
   if (act == 1) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
   return z / (1.0f + expf(-z));
+}
+
+// eight consecutive entries as floats
+template <typename V>
+__device__ __forceinline__ void ex_load8f(const V* p, float* out) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = to_f32(p[e]);
+}
+template <>
+__device__ __forceinline__ void ex_load8f<bf16_t>(const bf16_t* p, float* out) {
+  typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 v8;
+  const v8 v = *reinterpret_cast<const v8*>(p);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = (float)v[e];
+}
+template <>
+__device__ __forceinline__ void ex_load8f<float>(const float* p, float* out) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w; out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
 }
 
 // u[t * top + j, f] for the pair (t, j): one wave per f.
@@ -89,10 +90,24 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
   const T* g = gate_up + ((size_t)e * 2 * F + f) * W;
   const T* p = g + (size_t)F * W;
   float sg = 0.f, su = 0.f;
-  for (int k = lane; k < W; k += NHV_WAVE) {
-    const float xv = to_f32(x[k]);
-    sg = fmaf(to_f32(g[k]), xv, sg);
-    su = fmaf(to_f32(p[k]), xv, su);
+  if (W % 8 == 0) {                          // (rows then start at multiples of 16 or 32 bytes)
+    for (int k = lane * 8; k < W; k += NHV_WAVE * 8) {
+      float xv[8], gv[8], pv[8];
+      ex_load8f(x + k, xv);
+      ex_load8f(g + k, gv);
+      ex_load8f(p + k, pv);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        sg = fmaf(gv[i], xv[i], sg);
+        su = fmaf(pv[i], xv[i], su);
+      }
+    }
+  } else {
+    for (int k = lane; k < W; k += NHV_WAVE) {
+      const float xv = to_f32(x[k]);
+      sg = fmaf(to_f32(g[k]), xv, sg);
+      su = fmaf(to_f32(p[k]), xv, su);
+    }
   }
   sg = wave_sum(sg);
   su = wave_sum(su);
@@ -136,7 +151,17 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__
     const T* d = down + ((size_t)e * W + n) * F;
     const T* x = u + ((size_t)t * top + j) * F;
     float s = 0.f;
-    for (int f = lane; f < F; f += NHV_WAVE) s = fmaf(to_f32(d[f]), to_f32(x[f]), s);
+    if (F % 8 == 0) {
+      for (int f = lane * 8; f < F; f += NHV_WAVE * 8) {
+        float dv[8], xv[8];
+        ex_load8f(d + f, dv);
+        ex_load8f(x + f, xv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s = fmaf(dv[i], xv[i], s);
+      }
+    } else {
+      for (int f = lane; f < F; f += NHV_WAVE) s = fmaf(to_f32(d[f]), to_f32(x[f]), s);
+    }
     total += wave_sum(s);
   }
   if (lane == 0) out[(size_t)t * W + n] = from_f32<T>(total);
@@ -157,5 +182,226 @@ extern "C" int nhv_experts_down(const void* u, const void* ids, const void* down
   else
     return nhv_fail("experts_down: unknown dtype %d", dtype);
   NHV_LAUNCH_CHECK("experts_down");
+  return 0;
+}
+
+// ---------------------------------------------------------------- many rows in bfloat16: the pairs sorted by expert
+// The (token, expert) pairs of a step are put in the order of their experts, every expert's run filled up to whole
+// tiles of TM pairs (-1 where there is none), so that a block meets one expert's matrices only: nhv_experts_sort.
+// nhv_experts_grouped_gate_up and nhv_experts_grouped_down are then matrix products on the matrix cores in which a
+// block owns one tile of pairs and some tiles of 16 outputs; its waves share the inner dimension and their sums meet
+// in LDS in the order of the waves. A pair's sums do not depend on where the sort has put it.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+__device__ __forceinline__ bf16x8 ex_load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ bf16x8 ex_zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
+  return z;
+}
+
+// One block. sorted [cap]: the pair at each place, -1 for none; tile_expert [tiles_cap]: the expert of each tile of
+// TM places, -1 for a tile beyond the last.
+__global__ __launch_bounds__(1024) void experts_sort_kernel(const int* __restrict__ ids, int P, int E, int TM,
+                                                            int* __restrict__ sorted, int cap,
+                                                            int* __restrict__ tile_expert, int tiles_cap) {
+  extern __shared__ int sh[];                // counts [E], offsets [E], cursors [E]
+  int* counts = sh;
+  int* offsets = sh + E;
+  int* cursors = sh + 2 * E;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) { counts[e] = 0; cursors[e] = 0; }
+  for (int i = threadIdx.x; i < cap; i += blockDim.x) sorted[i] = -1;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = ids[p];
+    if (e >= 0 && e < E) atomicAdd(&counts[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int tile = 0;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = tile * TM;
+      const int n = (counts[e] + TM - 1) / TM;
+      for (int i = 0; i < n && tile < tiles_cap; ++i) tile_expert[tile++] = e;
+    }
+    for (; tile < tiles_cap; ++tile) tile_expert[tile] = -1;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = ids[p];
+    if (e >= 0 && e < E) {
+      const int at = offsets[e] + atomicAdd(&cursors[e], 1);
+      if (at < cap) sorted[at] = p;
+    }
+  }
+}
+
+extern "C" int nhv_experts_sort(const void* ids, int P, int E, int TM, void* sorted, int cap, void* tile_expert,
+                                int tiles_cap, void* stream) {
+  NHV_REQUIRE(P > 0 && E > 0 && E <= 4096 && TM > 0, "experts_sort: bad sizes P=%d E=%d TM=%d", P, E, TM);
+  NHV_REQUIRE(tiles_cap >= (P + TM - 1) / TM + E && cap >= tiles_cap * TM,
+              "experts_sort: room for %d tiles and %d places is too little for %d pairs of %d experts", tiles_cap, cap, P, E);
+  hipLaunchKernelGGL(experts_sort_kernel, dim3(1), dim3(1024), 3 * (size_t)E * sizeof(int), (hipStream_t)stream,
+                     (const int*)ids, P, E, TM, (int*)sorted, cap, (int*)tile_expert, tiles_cap);
+  NHV_LAUNCH_CHECK("experts_sort");
+  return 0;
+}
+
+// x: GLU: the step's rows [tokens, K] (pair p reads row p / top); else one row per pair [pairs, K]. w: [experts, NA N, K].
+// y: one row per pair [pairs, N]. GLU: y = act(s g) * (s u) with the pair's score s.
+template <int MT, int NT, int WAVES, int UNROLL, bool GLU, typename TOut>
+__global__ __launch_bounds__(64 * WAVES) void experts_grouped_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                                     TOut* __restrict__ y, const int* __restrict__ sorted,
+                                                                     const int* __restrict__ tile_expert,
+                                                                     const float* __restrict__ scores, int top, int N, int K,
+                                                                     int act) {
+  constexpr int NA = GLU ? 2 : 1;
+  constexpr int TILES = NA * NT;
+  static_assert(MT <= WAVES, "each of the first MT waves finishes one tile of rows");
+  __shared__ float red[WAVES][MT][4][64];
+  const int e = tile_expert[blockIdx.x];
+  if (e < 0) return;                         // the same for the whole block
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int n0 = blockIdx.y * 16 * NT;
+  const bf16_t* wbase = w + (size_t)e * NA * N * K;
+  const bf16_t* wrow[TILES];
+  bool n_ok[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int n = n0 + nt * 16 + col;
+    n_ok[nt] = n < N;
+#pragma unroll
+    for (int na = 0; na < NA; ++na) wrow[na * NT + nt] = wbase + ((size_t)na * N + (n_ok[nt] ? n : 0)) * K;
+  }
+  const int* places = sorted + (size_t)blockIdx.x * 16 * MT;
+  const bf16_t* xrow[MT];
+  bool m_ok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int pair = places[mt * 16 + col];
+    m_ok[mt] = pair >= 0;
+    xrow[mt] = x + (size_t)(m_ok[mt] ? (GLU ? pair / top : pair) : 0) * K;
+  }
+  floatx4 acc[TILES][MT];
+#pragma unroll
+  for (int t = 0; t < TILES; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int ksteps = (K + 31) / 32;
+  for (int run = wave; run * UNROLL < ksteps; run += WAVES) {
+    bf16x8 a[UNROLL][TILES], b[UNROLL][MT];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int k = (run * UNROLL + u) * 32 + grp * 8;
+      const bool k_ok = k < K;
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) a[u][t] = (n_ok[t % NT] && k_ok) ? ex_load8(wrow[t] + k) : ex_zero8();
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) b[u][mt] = (m_ok[mt] && k_ok) ? ex_load8(xrow[mt] + k) : ex_zero8();
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][t], b[u][mt], acc[t][mt], 0, 0, 0);
+  }
+  // wave ``mt`` adds the waves' partial sums of tile (nt, mt) in the order of the waves and writes that tile
+  const int my_pair = wave < MT ? places[wave * 16 + col] : -1;
+  const float s = (GLU && my_pair >= 0) ? scores[my_pair] : 1.0f;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    float v[NA][4];
+#pragma unroll
+    for (int na = 0; na < NA; ++na) {
+      __syncthreads();
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) red[wave][mt][j][lane] = acc[na * NT + nt][mt][j];
+      __syncthreads();
+      if (wave < MT) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float sum = 0.f;
+#pragma unroll
+          for (int wv = 0; wv < WAVES; ++wv) sum += red[wv][wave][j][lane];
+          v[na][j] = sum;
+        }
+      }
+    }
+    if (wave < MT && my_pair >= 0) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + nt * 16 + grp * 4 + j;
+        if (n < N) {
+          float r = v[0][j];
+          if (GLU) r = nhv_expert_act(s * r, act) * (s * v[NA - 1][j]);
+          y[(size_t)my_pair * N + n] = (TOut)r;
+        }
+      }
+    }
+  }
+}
+
+template <int MT, bool GLU, typename TOut>
+static void grouped_launch(hipStream_t s, const void* x, const void* w, void* y, const void* sorted, const void* tile_expert,
+                           const void* scores, int top, int N, int K, int act, int tiles_cap) {
+  constexpr int NT = GLU ? 2 : 4, WAVES = 8, UNROLL = 2;
+  const dim3 grid(tiles_cap, (N + 16 * NT - 1) / (16 * NT));
+  hipLaunchKernelGGL((experts_grouped_kernel<MT, NT, WAVES, UNROLL, GLU, TOut>), grid, dim3(64 * WAVES), 0, s,
+                     (const bf16_t*)x, (const bf16_t*)w, (TOut*)y, (const int*)sorted, (const int*)tile_expert,
+                     (const float*)scores, top, N, K, act);
+}
+
+// u [pairs, F] bfloat16 from the step's rows h [tokens, W]; TM: 16 or 64 places a tile (as the sort was told).
+extern "C" int nhv_experts_grouped_gate_up(const void* h, const void* gate_up, void* u, const void* sorted,
+                                           const void* tile_expert, const void* scores, int top, int W, int F, int act,
+                                           int TM, int tiles_cap, void* stream) {
+  NHV_REQUIRE(W > 0 && F > 0 && W % 8 == 0 && top > 0 && tiles_cap > 0 && (TM == 16 || TM == 64),
+              "experts_grouped_gate_up: bad sizes W=%d (a multiple of 8) F=%d top=%d TM=%d", W, F, top, TM);
+  NHV_REQUIRE((F + 31) / 32 <= 65535, "experts_grouped_gate_up: F=%d is beyond this kernel's grid", F);
+  hipStream_t s = (hipStream_t)stream;
+  if (TM == 64) grouped_launch<4, true, bf16_t>(s, h, gate_up, u, sorted, tile_expert, scores, top, F, W, act, tiles_cap);
+  else grouped_launch<1, true, bf16_t>(s, h, gate_up, u, sorted, tile_expert, scores, top, F, W, act, tiles_cap);
+  NHV_LAUNCH_CHECK("experts_grouped_gate_up");
+  return 0;
+}
+
+// y [pairs, W] float from u [pairs, F] bfloat16.
+extern "C" int nhv_experts_grouped_down(const void* u, const void* down, void* y, const void* sorted,
+                                        const void* tile_expert, int W, int F, int TM, int tiles_cap, void* stream) {
+  NHV_REQUIRE(W > 0 && F > 0 && F % 8 == 0 && tiles_cap > 0 && (TM == 16 || TM == 64),
+              "experts_grouped_down: bad sizes W=%d F=%d (a multiple of 8) TM=%d", W, F, TM);
+  NHV_REQUIRE((W + 63) / 64 <= 65535, "experts_grouped_down: W=%d is beyond this kernel's grid", W);
+  hipStream_t s = (hipStream_t)stream;
+  if (TM == 64) grouped_launch<4, false, float>(s, u, down, y, sorted, tile_expert, nullptr, 1, W, F, 0, tiles_cap);
+  else grouped_launch<1, false, float>(s, u, down, y, sorted, tile_expert, nullptr, 1, W, F, 0, tiles_cap);
+  NHV_LAUNCH_CHECK("experts_grouped_down");
+  return 0;
+}
+
+// out[t, n] = sum over j < top (rising) of y[t * top + j, n]
+__global__ void experts_combine_kernel(const float* __restrict__ y, bf16_t* __restrict__ out, int W, int top, size_t total) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = i / W, n = i % W;
+    float sum = 0.f;
+    for (int j = 0; j < top; ++j) sum += y[(t * top + j) * W + n];
+    out[i] = (bf16_t)sum;
+  }
+}
+
+extern "C" int nhv_experts_combine(const void* y, void* out, int T, int W, int top, void* stream) {
+  NHV_REQUIRE(T > 0 && W > 0 && top > 0, "experts_combine: bad sizes T=%d W=%d top=%d", T, W, top);
+  const size_t total = (size_t)T * W;
+  const int blocks = (int)((total + 255) / 256 > 65535 * 4 ? 65535 * 4 : (total + 255) / 256);
+  hipLaunchKernelGGL(experts_combine_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const float*)y, (bf16_t*)out,
+                     W, top, total);
+  NHV_LAUNCH_CHECK("experts_combine");
   return 0;
 }

@@ -273,22 +273,32 @@ class NativeBackend:
                    ctypes.c_float(eps), _ptr(freqs), ctypes.c_float(gain), _ptr(positions), _ptr(slot_mapping), _ptr(cache),
                    0 if cache is None else cache.shape[-1], _ptr(cq), a.shape[0], dtype_code(cq), _stream())
 
-    def head_gemm(self, x, x_off, x_row, w, w_head, w_n, w_k, y, y_off, y_row, gate, gate_off, N, K):
-        """y[t, h, y_off : y_off + N] = M_h x[t, h, x_off : x_off + K]; x and y are [rows, heads, x_row / y_row]."""
+    def head_gemm(self, x, x_off, x_row, w, w_head, w_n, w_k, y, y_off, y_row, gate, gate_off, N, K, turn=None):
+        """y[t, h, y_off : y_off + N] = M_h x[t, h, x_off : x_off + K]; x and y are [rows, heads, x_row / y_row].
+        ``turn`` = (rot, x_rot_off, y_rot_off, freqs, gain, positions): also y[t, h, y_rot_off ...] = the ``rot`` entries
+        of x from x_rot_off on, turned. Returns whether the turning was done (up to 16 rows: in the same launch)."""
         T, H = x.shape[0], x.shape[1]
         item = x.element_size()
         LL = ctypes.c_longlong
         gate_p = None if gate is None else ctypes.c_void_p(gate.data_ptr() + 4 * gate_off)
-        if x.dtype == torch.bfloat16 and T > self.few_rows and not self.own_kernels_only and gate is None:
+        x_p, y_p = ctypes.c_void_p(x.data_ptr() + item * x_off), ctypes.c_void_p(y.data_ptr() + item * y_off)
+        gs_t = LL(0 if gate is None else gate.shape[1])
+        if T <= 16 and K <= 1024:
+            rot, xr, yr, freqs, gain, positions = turn if turn is not None else (0, 0, 0, None, 1.0, None)
+            self._call("nhv_head_gemm_fewrows", x_p, LL(H * x_row), LL(x_row), _ptr(w), LL(w_head), LL(w_n), LL(w_k), y_p,
+                       LL(H * y_row), LL(y_row), gate_p, gs_t, T, H, N, K, rot, xr - x_off, yr - y_off, _ptr(freqs),
+                       ctypes.c_float(gain), _ptr(positions), dtype_code(x), _stream())
+            return True
+        if x.dtype == torch.bfloat16 and not self.own_kernels_only and gate is None:
             # many rows: the library's batched product, one matrix per head, on strided views
             xv = x[:, :, x_off:x_off + K].transpose(0, 1)                         # [H, T, K]
             wv = torch.as_strided(w, (H, K, N), (w_head, w_k, w_n))
             yv = y[:, :, y_off:y_off + N].transpose(0, 1)
             yv.copy_(torch.bmm(xv, wv))
-            return
-        self._call("nhv_head_gemm", ctypes.c_void_p(x.data_ptr() + item * x_off), LL(H * x_row), LL(x_row), _ptr(w),
-                   LL(w_head), LL(w_n), LL(w_k), ctypes.c_void_p(y.data_ptr() + item * y_off), LL(H * y_row), LL(y_row),
-                   gate_p, LL(0 if gate is None else gate.shape[1]), T, H, N, K, dtype_code(x), _stream())
+            return False
+        self._call("nhv_head_gemm", x_p, LL(H * x_row), LL(x_row), _ptr(w), LL(w_head), LL(w_n), LL(w_k), y_p, LL(H * y_row),
+                   LL(y_row), gate_p, gs_t, T, H, N, K, dtype_code(x), _stream())
+        return False
 
     def rotate_interleaved(self, src, s_off, dst, d_off, rot, freqs, gain, positions):
         T, H, s_row = src.shape
@@ -296,16 +306,35 @@ class NativeBackend:
                    ctypes.c_float(gain), _ptr(positions), T, H, dtype_code(src), _stream())
 
     # -- a feed-forward of many small experts --
-    def route_topk(self, h, router, ids, scores):
-        T, W = h.shape
-        self._call("nhv_route_topk", _ptr(h), _ptr(router), _ptr(ids), _ptr(scores), T, W, router.shape[0], ids.shape[1],
-                   dtype_code(h), _stream())
+    def route_topk(self, logits, ids, scores):
+        T, E = logits.shape
+        self._call("nhv_route_topk", _ptr(logits), _ptr(ids), _ptr(scores), T, E, ids.shape[1], _stream())
 
     def experts_gate_up(self, h, ids, scores, gate_up, u, act):
         T, W = h.shape
         E, F2, _ = gate_up.shape
         self._call("nhv_experts_gate_up", _ptr(h), _ptr(ids), _ptr(scores), _ptr(gate_up), _ptr(u), T, W, F2 // 2,
                    ids.shape[1], E, act, dtype_code(h), _stream())
+
+    def experts_grouped(self, h, ids, scores, gate_up, down, out, act):
+        """Many rows in bfloat16: the pairs sorted by expert, then both products on the matrix cores, then the sum over
+        a token's experts."""
+        T, W = h.shape
+        E, F2, _ = gate_up.shape
+        F, top = F2 // 2, ids.shape[1]
+        P = T * top
+        TM = 64 if P >= 32 * E else 16                  # places a tile: runs of an expert's pairs are filled up to whole tiles
+        tiles = -(-P // TM) + E
+        index = torch.empty(tiles * TM + tiles, dtype=torch.int32, device=h.device)
+        sorted_pairs, tile_expert = index[:tiles * TM], index[tiles * TM:]
+        self._call("nhv_experts_sort", _ptr(ids), P, E, TM, _ptr(sorted_pairs), tiles * TM, _ptr(tile_expert), tiles, _stream())
+        u = torch.empty((P, F), dtype=h.dtype, device=h.device)
+        self._call("nhv_experts_grouped_gate_up", _ptr(h), _ptr(gate_up), _ptr(u), _ptr(sorted_pairs), _ptr(tile_expert),
+                   _ptr(scores), top, W, F, act, TM, tiles, _stream())
+        y = torch.empty((P, W), dtype=torch.float32, device=h.device)
+        self._call("nhv_experts_grouped_down", _ptr(u), _ptr(down), _ptr(y), _ptr(sorted_pairs), _ptr(tile_expert), W, F, TM,
+                   tiles, _stream())
+        self._call("nhv_experts_combine", _ptr(y), _ptr(out), T, W, top, _stream())
 
     def experts_down(self, u, ids, down, out):
         T, W = out.shape
@@ -1180,11 +1209,13 @@ def latent_prepare(a: torch.Tensor, q_off: int, q_rank: int, c_off: int, kv_rank
 
 
 def head_gemm(x: torch.Tensor, w: torch.Tensor, transposed: bool, N: int, K: int, x_off: int = 0, out: torch.Tensor | None = None,
-              out_off: int = 0, gate: torch.Tensor | None = None, gate_off: int = 0) -> torch.Tensor:
+              out_off: int = 0, gate: torch.Tensor | None = None, gate_off: int = 0, turn: tuple | None = None) -> torch.Tensor:
     """One small matrix per head: out[t, h, out_off : out_off + N] = M_h x[t, h, x_off : x_off + K], sums in float.
     ``w`` is [heads * K, N] with M_h = w[h K : (h + 1) K]^T (``transposed``: x is multiplied from the left by the
     block's transpose) or [heads * N, K] with M_h = w[h N : (h + 1) N]. ``gate`` [tokens, columns] float32: the result
-    of (t, h) is multiplied by sigmoid(gate[t, gate_off + h]). ``out``: [tokens, heads, row] to write into."""
+    of (t, h) is multiplied by sigmoid(gate[t, gate_off + h]). ``out``: [tokens, heads, row] to write into.
+    ``turn`` = (rot, x_rot_off, out_rot_off, freqs, gain, positions): also out[t, h, out_rot_off + j] = x[t, h,
+    x_rot_off + j] turned, j < rot, as ``rotate_interleaved`` does (for few rows in the same launch)."""
     _need(x.dim() == 3, "head_gemm: x must be [tokens, heads, row]")
     T, H, x_row = x.shape
     _dense(x, "head_gemm: x")
@@ -1204,7 +1235,18 @@ def head_gemm(x: torch.Tensor, w: torch.Tensor, transposed: bool, N: int, K: int
         w_head, w_n, w_k = K * N, 1, N
     else:
         w_head, w_n, w_k = N * K, K, 1
-    backend().head_gemm(x, x_off, x_row, w, w_head, w_n, w_k, out, out_off, out.shape[2], gate, gate_off, N, K)
+    if turn is None:
+        backend().head_gemm(x, x_off, x_row, w, w_head, w_n, w_k, out, out_off, out.shape[2], gate, gate_off, N, K)
+        return out
+    rot, x_rot, out_rot, freqs, gain, positions = turn
+    _need(rot > 0 and rot % 2 == 0 and 0 <= x_rot and x_rot + rot <= x_row and 0 <= out_rot and out_rot + rot <= out.shape[2],
+          lambda: f"head_gemm: {rot} turned entries at {x_rot} of {x_row} into {out_rot} of {out.shape[2]}")
+    _dense(freqs, "head_gemm: frequencies", (rot // 2,), torch.float64)
+    _dense(positions, "head_gemm: positions", (T,), torch.int32)
+    done = backend().head_gemm(x, x_off, x_row, w, w_head, w_n, w_k, out, out_off, out.shape[2], gate, gate_off, N, K,
+                               turn=(rot, x_rot, out_rot, freqs, float(gain), positions))
+    if not done:
+        backend().rotate_interleaved(x, x_rot, out, out_rot, rot, freqs, float(gain), positions)
     return out
 
 
@@ -1225,18 +1267,15 @@ def rotate_interleaved(src: torch.Tensor, s_off: int, dst: torch.Tensor, d_off: 
 
 
 # ------------------------------------------------------------------ a feed-forward of many small experts
-def route_topk(h: torch.Tensor, router: torch.Tensor, top: int):
-    """(numbers [tokens, top] int32, scores [tokens, top] float32) of the ``top`` experts with the largest
-    sigmoid(router . h), logits summed in float; the largest first, the lower number among equals."""
-    _need(h.dim() == 2, "route_topk: h must be [tokens, width]")
-    _dense(h, "route_topk: h")
-    dtype_code(h)
-    _need(router.dim() == 2, "route_topk: the router must be [experts, width]")
-    _float32(router, "route_topk: router", (router.shape[0], h.shape[1]))
-    _need(0 < top <= router.shape[0], lambda: f"route_topk: {top} of {router.shape[0]} experts")
-    ids = torch.empty((h.shape[0], top), dtype=torch.int32, device=h.device)
-    scores = torch.empty((h.shape[0], top), dtype=torch.float32, device=h.device)
-    backend().route_topk(h, router, ids, scores)
+def route_topk(logits: torch.Tensor, top: int):
+    """(numbers [tokens, top] int32, scores [tokens, top] float32) of the ``top`` experts with the largest logits, the
+    largest first, the lower number among equals; a score is the sigmoid of its logit."""
+    _need(logits.dim() == 2, "route_topk: logits must be [tokens, experts]")
+    _dense(logits, "route_topk: logits", dtype=torch.float32)
+    _need(0 < top <= logits.shape[1], lambda: f"route_topk: {top} of {logits.shape[1]} experts")
+    ids = torch.empty((logits.shape[0], top), dtype=torch.int32, device=logits.device)
+    scores = torch.empty((logits.shape[0], top), dtype=torch.float32, device=logits.device)
+    backend().route_topk(logits, ids, scores)
     return ids, scores
 
 
@@ -1256,10 +1295,15 @@ def routed_experts(h: torch.Tensor, ids: torch.Tensor, scores: torch.Tensor, gat
     _need(ids.dim() == 2 and ids.shape[0] == T, "routed_experts: ids must be [tokens, top]")
     _dense(ids, "routed_experts: ids", dtype=torch.int32)
     _dense(scores, "routed_experts: scores", tuple(ids.shape), torch.float32)
-    u = torch.empty((T * ids.shape[1], F), dtype=h.dtype, device=h.device)
-    backend().experts_gate_up(h, ids, scores, gate_up, u, ACTIVATIONS[activation])
     out = torch.empty((T, W), dtype=h.dtype, device=h.device)
-    backend().experts_down(u, ids, down, out)
+    b = backend()
+    if (h.dtype == torch.bfloat16 and T > getattr(b, "few_rows", 0) and W % 8 == 0 and F % 8 == 0 and E <= 4096
+            and hasattr(b, "experts_grouped")):
+        b.experts_grouped(h, ids, scores, gate_up, down, out, ACTIVATIONS[activation])
+        return out
+    u = torch.empty((T * ids.shape[1], F), dtype=h.dtype, device=h.device)
+    b.experts_gate_up(h, ids, scores, gate_up, u, ACTIVATIONS[activation])
+    b.experts_down(u, ids, down, out)
     return out
 
 # ------------------------------------------------------------------ layers that are not the pre-norm kind

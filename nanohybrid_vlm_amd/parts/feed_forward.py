@@ -45,7 +45,7 @@ class SwiGLU(Part):
 @FEED_FORWARDS.register("routed_experts")
 class RoutedExperts(Part):
     """``num_experts`` gated feed-forwards of inner size ``expert_size`` without biases, of which every token uses the
-    ``top`` with the largest score s_e = sigmoid(router_e . x) (logits in float32). The scores are taken as they are
+    ``top`` with the largest score s_e = sigmoid(router_e . x) (the logits are summed and kept in float32). The scores are taken as they are
     (not renormalised) and multiply the experts' inputs: y = sum over chosen e of D_e (act(G_e s_e x) * (U_e s_e x)).
     All experts' matrices lie in two tensors, [experts * 2 expert_size, width] (per expert its gate rows, then its
     up rows) and [experts * width, expert_size]."""
@@ -60,7 +60,7 @@ class RoutedExperts(Part):
 
     def param_specs(self):
         E, F, W = self.num_experts, self.expert_size, self.hidden_size
-        return {"router.weight": ParamSpec((E, W), always_float32=True),
+        return {"router.weight": ParamSpec((E, W)),
                 "gate_up.weight": ParamSpec((E * 2 * F, W)),
                 "down.weight": ParamSpec((E * W, F))}
 
@@ -71,5 +71,5 @@ class RoutedExperts(Part):
         self.down_weight = params["down.weight"].view(E, W, F)
 
     def forward(self, x, step):
-        ids, scores = ops.route_topk(x, self.router_weight, self.top)
+        ids, scores = ops.route_topk(ops.linear(x, self.router_weight, out_dtype=torch.float32), self.top)
         return ops.routed_experts(x, ids, scores, self.gate_up_weight, self.down_weight, self.activation)

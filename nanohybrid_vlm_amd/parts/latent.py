@@ -80,9 +80,8 @@ class LatentAttention(Part):
         # the query as the stored rows see it: [W_uk,h^T q_h' | q_h'' turned | zeros]
         make = torch.zeros if self.pad_dim else torch.empty
         q_row = make((T, H, self.row), dtype=x.dtype, device=x.device)
-        ops.head_gemm(q, self.uk_weight, True, self.kv_rank, D, out=q_row)
-        if R:
-            ops.rotate_interleaved(q, D, q_row, self.kv_rank, R, freqs, gain, step.token_positions)
+        ops.head_gemm(q, self.uk_weight, True, self.kv_rank, D, out=q_row,
+                      turn=(R, D, self.kv_rank, freqs, gain, step.token_positions) if R else None)
         mixed = ops.paged_attention(q_row, cache.k, cache.k, step.attention, tables.block_tables, self.scale)
         o = ops.head_gemm(mixed, self.uv_weight, False, self.value_dim, self.kv_rank,
                           gate=a if self.gated else None, gate_off=self.gate_off)

@@ -198,24 +198,23 @@ class EmulatedBackend:
         ok = slot_mapping >= 0
         cache.view(-1, cache.shape[-1])[slot_mapping[ok].long(), :kv_rank + rot] = rows[ok]
 
-    def head_gemm(self, x, x_off, x_row, w, w_head, w_n, w_k, y, y_off, y_row, gate, gate_off, N, K):
+    def head_gemm(self, x, x_off, x_row, w, w_head, w_n, w_k, y, y_off, y_row, gate, gate_off, N, K, turn=None):
         T, H = x.shape[0], x.shape[1]
         m = torch.as_strided(w, (H, N, K), (w_head, w_n, w_k)).float()
         r = torch.einsum("thk,hnk->thn", x[:, :, x_off:x_off + K].float(), m)
         if gate is not None:
             r = r * torch.sigmoid(gate[:, gate_off:gate_off + H])[:, :, None]
         y[:, :, y_off:y_off + N] = r.to(y.dtype)
+        return False                               # (the turning is left to rotate_interleaved)
 
     def rotate_interleaved(self, src, s_off, dst, d_off, rot, freqs, gain, positions):
         dst[:, :, d_off:d_off + rot] = self._turn_pairs(src[:, :, s_off:s_off + rot].float(), positions, freqs, gain).to(dst.dtype)
 
     # -- a feed-forward of many small experts
-    def route_topk(self, h, router, ids, scores):
-        z = h.float() @ router.T
-        top = ids.shape[1]
-        order = torch.sort(z, dim=-1, descending=True, stable=True).indices[:, :top]
+    def route_topk(self, logits, ids, scores):
+        order = torch.sort(logits, dim=-1, descending=True, stable=True).indices[:, :ids.shape[1]]
         ids.copy_(order.to(torch.int32))
-        scores.copy_(torch.sigmoid(torch.gather(z, 1, order)))
+        scores.copy_(torch.sigmoid(torch.gather(logits, 1, order)))
 
     def experts_gate_up(self, h, ids, scores, gate_up, u, act):
         T, top = ids.shape

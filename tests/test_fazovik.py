@@ -241,7 +241,8 @@ def test_routed_experts_alone(where, kernels):
     device, dtype = where
     dt = _dt(dtype)
     g = torch.Generator().manual_seed(8)
-    for E, top, F, W, T in ((5, 2, 12, 20, 9), (1, 1, 8, 16, 3), (7, 7, 4, 12, 4), (70, 3, 8, 24, 21)):
+    for E, top, F, W, T in ((5, 2, 12, 20, 9), (1, 1, 8, 16, 3), (7, 7, 4, 12, 4), (70, 3, 8, 24, 21), (2, 1, 16, 32, 70),
+                            (3, 2, 24, 40, 130)):
         w = {"router": (torch.randn(E, W, generator=g) * 0.6).to(torch.bfloat16).double()}
         for e in range(E):
             w[f"e{e}.gate"] = (torch.randn(F, W, generator=g) / W ** 0.5).to(torch.bfloat16).double()
@@ -249,7 +250,8 @@ def test_routed_experts_alone(where, kernels):
             w[f"e{e}.down"] = (torch.randn(W, F, generator=g) / F ** 0.5).to(torch.bfloat16).double()
         h = torch.randn(T, W, generator=g).to(torch.bfloat16)
         want = plain.routed_ff(h.double(), w, "", {"router": {"experts": E, "top": top}}).float()
-        ids, scores = ops.route_topk(h.to(dt).to(device), w["router"].float().to(device), top)
+        logits = ops.linear(h.to(dt).to(device), w["router"].to(dt).to(device), out_dtype=torch.float32)
+        ids, scores = ops.route_topk(logits, top)
         s = torch.sigmoid(h.double() @ w["router"].T)
         assert torch.equal(ids.cpu().long().sort(dim=-1).values, torch.topk(s, top, dim=-1).indices.sort(dim=-1).values)
         assert max_abs_diff(scores.cpu(), torch.gather(s, 1, ids.cpu().long()).float()) < 1e-5
