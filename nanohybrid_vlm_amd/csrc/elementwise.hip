@@ -1,4 +1,4 @@
-// Embedding gather, RMSNorm (+ residual add), SiLU-and-multiply, row gather and
+// Embedding gather, RMSNorm (+ residual add), SiLU- or GELU-and-multiply, row gather and
 // the fused q/k-norm + rotation + cache-write kernel. All in two element types
 // (float, bfloat16); statistics, angles and sums are float.
 #include "nhv_common.h"
@@ -186,20 +186,27 @@ extern "C" int nhv_rmsnorm(const void* x, void* residual, int residual_mode, int
   return 0;
 }
 
-// ---------------------------------------------------------------- SiLU(gate) * up
+// ---------------------------------------------------------------- act(gate) * up
 // gu: [T, 2I], gate = first I columns, up = last I. Float inside, rounded once.
-template <typename T>
+// act 0: SiLU, z sigmoid(z). act 1: GELU in its tanh form, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).
+template <int ACT>
+__device__ __forceinline__ float gate_act(float z) {
+  if (ACT == 1) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return z / (1.0f + expf(-z));
+}
+
+template <typename T, int ACT = 0>
 __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
     const size_t t = idx / I, i = idx % I;
     const float g = to_f32(gu[t * 2 * I + i]);
     const float u = to_f32(gu[t * 2 * I + I + i]);
-    out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+    out[idx] = from_f32<T>(gate_act<ACT>(g) * u);
   }
 }
 
 // the same, eight entries a thread (widths that are a multiple of 8)
-template <typename T>
+template <typename T, int ACT = 0>
 __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total8) {
   const int per_row = I / 8;
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total8; idx += (size_t)gridDim.x * blockDim.x) {
@@ -208,7 +215,7 @@ __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ ou
     load8f<T>(gu + t * 2 * I + c * 8, g);
     load8f<T>(gu + t * 2 * I + I + c * 8, u);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) o[e] = g[e] / (1.0f + expf(-g[e])) * u[e];
+    for (int e = 0; e < 8; ++e) o[e] = gate_act<ACT>(g[e]) * u[e];
     store8f<T>(out + t * I + c * 8, o);
   }
 }
@@ -238,6 +245,35 @@ extern "C" int nhv_silu_mul(const void* gu, void* out, int T, int I, int dtype, 
   else
     return nhv_fail("silu_mul: unknown dtype %d", dtype);
   NHV_LAUNCH_CHECK("silu_mul");
+  return 0;
+}
+
+// the same with the tanh form of GELU on the gate
+extern "C" int nhv_gelu_tanh_mul(const void* gu, void* out, int T, int I, int dtype, void* stream) {
+  NHV_REQUIRE(T > 0 && I > 0, "gelu_tanh_mul: bad sizes T=%d I=%d", T, I);
+  if (I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    const size_t total8 = (size_t)T * (I / 8);
+    const int vblocks = (int)((total8 + 255) / 256 > 65535 * 16 ? 65535 * 16 : (total8 + 255) / 256);
+    hipStream_t vs = (hipStream_t)stream;
+    if (dtype == NHV_F32)
+      hipLaunchKernelGGL((silu_mul_vec_kernel<float, 1>), dim3(vblocks), dim3(256), 0, vs, (const float*)gu, (float*)out, I, total8);
+    else if (dtype == NHV_BF16)
+      hipLaunchKernelGGL((silu_mul_vec_kernel<bf16_t, 1>), dim3(vblocks), dim3(256), 0, vs, (const bf16_t*)gu, (bf16_t*)out, I, total8);
+    else
+      return nhv_fail("gelu_tanh_mul: unknown dtype %d", dtype);
+    NHV_LAUNCH_CHECK("gelu_tanh_mul");
+    return 0;
+  }
+  const size_t total = (size_t)T * I;
+  const int blocks = (int)((total + 255) / 256 > 65535 * 4 ? 65535 * 4 : (total + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == NHV_F32)
+    hipLaunchKernelGGL((silu_mul_kernel<float, 1>), dim3(blocks), dim3(256), 0, s, (const float*)gu, (float*)out, I, total);
+  else if (dtype == NHV_BF16)
+    hipLaunchKernelGGL((silu_mul_kernel<bf16_t, 1>), dim3(blocks), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)out, I, total);
+  else
+    return nhv_fail("gelu_tanh_mul: unknown dtype %d", dtype);
+  NHV_LAUNCH_CHECK("gelu_tanh_mul");
   return 0;
 }
 

@@ -162,10 +162,12 @@ extern "C" int nhv_head_gemm(const void* x, long long xs_t, long long xs_h, cons
   return 0;
 }
 
-// The same for up to 16 rows (a decoding step): a block owns 256 outputs of one head, keeps the head's rows of x in LDS
-// as floats and gives every thread one output of all rows; k rises as above, so the sums are the same bits. One more
-// block a head may turn the rotated part of x and copy it beside the outputs (``rot`` entries from x_rot_off to
-// y_rot_off), which saves the launch of nhv_rotate_interleaved.
+// The same for up to 16 rows (a decoding step): a block owns 64 outputs of one head. It first brings the head's rows
+// of x (as floats) and its 64 x K piece of the matrix into LDS, every thread asking for all its share at once (a
+// thread that walked over k with loads from memory waited for memory at every step); then lane = output, wave = four
+// of the rows, k rising as above, so the sums are the same bits. One more block a head may turn the rotated part of x
+// and copy it beside the outputs (``rot`` entries from x_rot_off to y_rot_off), which saves the launch of
+// nhv_rotate_interleaved.
 template <typename T>
 __global__ __launch_bounds__(256) void head_gemm_fewrows_kernel(const T* __restrict__ x, long long xs_t, long long xs_h,
                                                                 const T* __restrict__ w, long long ws_h, long long ws_n,
@@ -174,7 +176,7 @@ __global__ __launch_bounds__(256) void head_gemm_fewrows_kernel(const T* __restr
                                                                 long long gs_t, int rows, int N, int K, int n_chunks, int rot,
                                                                 int x_rot_off, int y_rot_off, const double* __restrict__ freqs,
                                                                 float gain, const int* __restrict__ positions) {
-  extern __shared__ float xs[];              // 16 x K
+  extern __shared__ float xs[];              // 16 x K floats, then the block's piece of the matrix
   const int h = blockIdx.y;
   if ((int)blockIdx.x == n_chunks) {         // the rotated part
     for (int i = threadIdx.x; i < rows * (rot / 2); i += blockDim.x) {
@@ -189,28 +191,44 @@ __global__ __launch_bounds__(256) void head_gemm_fewrows_kernel(const T* __restr
     }
     return;
   }
+  // [K][LDW]: rows one bank longer than 64 outputs, so that threads that walk along k (a matrix that is contiguous in k)
+  // store into different banks
+  constexpr int LDW = 64 + 4 / (int)sizeof(T);
+  T* wl = reinterpret_cast<T*>(xs + 16 * K);
+  const int n0 = blockIdx.x * 64;
+  const T* wh = w + (size_t)h * ws_h;
+  if (ws_k == 1) {                           // a row of the matrix is contiguous in k: threads walk along k
+    for (int i = threadIdx.x; i < 64 * K; i += blockDim.x) {
+      const int n = i / K, k = i % K;
+      wl[k * LDW + n] = n0 + n < N ? wh[(size_t)(n0 + n) * ws_n + k] : from_f32<T>(0.f);
+    }
+  } else {                                   // contiguous in n
+    for (int i = threadIdx.x; i < 64 * K; i += blockDim.x) {
+      const int k = i / 64, n = i % 64;
+      wl[k * LDW + n] = n0 + n < N ? wh[(size_t)(n0 + n) * ws_n + (size_t)k * ws_k] : from_f32<T>(0.f);
+    }
+  }
   for (int i = threadIdx.x; i < 16 * K; i += blockDim.x) {
     const int t = i / K, k = i % K;
     xs[i] = t < rows ? to_f32(x[(size_t)t * xs_t + (size_t)h * xs_h + k]) : 0.f;
   }
   __syncthreads();
-  const int n = blockIdx.x * 256 + threadIdx.x;
-  if (n >= N) return;
-  float acc[16];
-#pragma unroll
-  for (int t = 0; t < 16; ++t) acc[t] = 0.f;
-  const T* wn = w + (size_t)h * ws_h + (size_t)n * ws_n;
+  const int lane = threadIdx.x & 63, t0 = (threadIdx.x >> 6) * 4;
+  const int n = n0 + lane;
+  if (n >= N || t0 >= rows) return;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  const float* x0 = xs + t0 * K;
   for (int k = 0; k < K; ++k) {
-    const float wv = to_f32(wn[(size_t)k * ws_k]);
+    const float wv = to_f32(wl[k * LDW + lane]);
 #pragma unroll
-    for (int t = 0; t < 16; ++t) acc[t] = fmaf(xs[t * K + k], wv, acc[t]);
+    for (int t = 0; t < 4; ++t) acc[t] = fmaf(x0[t * K + k], wv, acc[t]);
   }
 #pragma unroll
-  for (int t = 0; t < 16; ++t) {
-    if (t >= rows) break;
+  for (int t = 0; t < 4; ++t) {
+    if (t0 + t >= rows) break;
     float v = acc[t];
-    if (gate != nullptr) v *= 1.0f / (1.0f + expf(-gate[(size_t)t * gs_t + h]));
-    y[(size_t)t * ys_t + (size_t)h * ys_h + n] = from_f32<T>(v);
+    if (gate != nullptr) v *= 1.0f / (1.0f + expf(-gate[(size_t)(t0 + t) * gs_t + h]));
+    y[(size_t)(t0 + t) * ys_t + (size_t)h * ys_h + n] = from_f32<T>(v);
   }
 }
 
@@ -218,25 +236,55 @@ extern "C" int nhv_head_gemm_fewrows(const void* x, long long xs_t, long long xs
                                      long long ws_n, long long ws_k, void* y, long long ys_t, long long ys_h, const void* gate,
                                      long long gs_t, int rows, int H, int N, int K, int rot, int x_rot_off, int y_rot_off,
                                      const void* freqs, float gain, const void* positions, int dtype, void* stream) {
-  NHV_REQUIRE(rows > 0 && rows <= 16 && H > 0 && H <= 65535 && N > 0 && K > 0 && K <= 1024,
-              "head_gemm_fewrows: bad sizes rows=%d (up to 16) H=%d N=%d K=%d (up to 1024)", rows, H, N, K);
+  const size_t item = dtype == NHV_F32 ? 4 : 2;
+  const size_t lds = 16 * (size_t)K * sizeof(float) + (64 + 4 / item) * (size_t)K * item;
+  NHV_REQUIRE(rows > 0 && rows <= 16 && H > 0 && H <= 65535 && N > 0 && K > 0 && lds <= 96 * 1024,
+              "head_gemm_fewrows: bad sizes rows=%d (up to 16) H=%d N=%d K=%d (LDS of %zu bytes, up to 98304)", rows, H, N, K, lds);
   NHV_REQUIRE(rot >= 0 && rot % 2 == 0 && (rot == 0 || (freqs != nullptr && positions != nullptr)),
               "head_gemm_fewrows: a rotated part of %d entries needs frequencies and positions", rot);
-  const int n_chunks = (N + 255) / 256;
+  const int n_chunks = (N + 63) / 64;
   const dim3 grid(n_chunks + (rot > 0 ? 1 : 0), H);
-  const size_t lds = 16 * (size_t)K * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == NHV_F32)
+  if (dtype == NHV_F32) {
+    if (lds > 64 * 1024) hipFuncSetAttribute((const void*)head_gemm_fewrows_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(head_gemm_fewrows_kernel<float>, grid, dim3(256), lds, s, (const float*)x, xs_t, xs_h, (const float*)w,
                        ws_h, ws_n, ws_k, (float*)y, ys_t, ys_h, (const float*)gate, gs_t, rows, N, K, n_chunks, rot, x_rot_off,
                        y_rot_off, (const double*)freqs, gain, (const int*)positions);
-  else if (dtype == NHV_BF16)
+  } else if (dtype == NHV_BF16) {
+    if (lds > 64 * 1024) hipFuncSetAttribute((const void*)head_gemm_fewrows_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(head_gemm_fewrows_kernel<bf16_t>, grid, dim3(256), lds, s, (const bf16_t*)x, xs_t, xs_h,
                        (const bf16_t*)w, ws_h, ws_n, ws_k, (bf16_t*)y, ys_t, ys_h, (const float*)gate, gs_t, rows, N, K,
                        n_chunks, rot, x_rot_off, y_rot_off, (const double*)freqs, gain, (const int*)positions);
-  else
+  } else {
     return nhv_fail("head_gemm_fewrows: unknown dtype %d", dtype);
+  }
   NHV_LAUNCH_CHECK("head_gemm_fewrows");
+  return 0;
+}
+
+// ---------------------------------------------------------------- the gate alone
+// y[t, h, :] *= sigmoid(gate[t * gs_t + h]) for rows that a library product has made
+template <typename T>
+__global__ void head_gate_kernel(T* __restrict__ y, const float* __restrict__ gate, long long gs_t, int H, int N, size_t total) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t th = i / N;
+    const float g = gate[(th / H) * gs_t + th % H];
+    y[i] = from_f32<T>(to_f32(y[i]) * (1.0f / (1.0f + expf(-g))));
+  }
+}
+
+extern "C" int nhv_head_gate(void* y, const void* gate, long long gs_t, int rows, int H, int N, int dtype, void* stream) {
+  NHV_REQUIRE(rows > 0 && H > 0 && N > 0 && gate != nullptr, "head_gate: bad sizes rows=%d H=%d N=%d", rows, H, N);
+  const size_t total = (size_t)rows * H * N;
+  const int blocks = (int)((total + 255) / 256 > 65535 * 4 ? 65535 * 4 : (total + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == NHV_F32)
+    hipLaunchKernelGGL(head_gate_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)y, (const float*)gate, gs_t, H, N, total);
+  else if (dtype == NHV_BF16)
+    hipLaunchKernelGGL(head_gate_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (bf16_t*)y, (const float*)gate, gs_t, H, N, total);
+  else
+    return nhv_fail("head_gate: unknown dtype %d", dtype);
+  NHV_LAUNCH_CHECK("head_gate");
   return 0;
 }
 

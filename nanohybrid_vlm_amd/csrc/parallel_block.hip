@@ -3,7 +3,6 @@
 //   nhv_embed_pair_hash   rows of two tables added in float; the previous token of a request is kept per state slot
 //   nhv_layernorm_pair    x (+ a + b) -> one or two layer norms (weight and bias) of it; x is the float stream
 //   nhv_add_streams       x += a (+ b)
-//   nhv_act_mul           act(gate) * up for a packed gate | up row; act: SiLU or the tanh form of GELU
 // Rows are float or bfloat16; the stream, statistics and sums are float.
 #include "nhv_common.h"
 #include <math.h>
@@ -142,38 +141,5 @@ extern "C" int nhv_add_streams(void* x, const void* a, const void* b, size_t n, 
   else
     return nhv_fail("add_streams: unknown dtype %d", dtype);
   NHV_LAUNCH_CHECK("add_streams");
-  return 0;
-}
-
-// ---------------------------------------------------------------- act(gate) * up
-// act 0: SiLU, z sigmoid(z). act 1: GELU in its tanh form, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).
-__device__ __forceinline__ float nhv_act(float z, int act) {
-  if (act == 1) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-  return z / (1.0f + expf(-z));
-}
-
-template <typename T>
-__global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total, int act) {
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-    const size_t t = i / I, c = i % I;
-    const float g = to_f32(gu[t * 2 * I + c]);
-    const float u = to_f32(gu[t * 2 * I + I + c]);
-    out[i] = from_f32<T>(nhv_act(g, act) * u);
-  }
-}
-
-extern "C" int nhv_act_mul(const void* gu, void* out, int T, int I, int act, int dtype, void* stream) {
-  NHV_REQUIRE(T > 0 && I > 0, "act_mul: bad sizes T=%d I=%d", T, I);
-  NHV_REQUIRE(act == 0 || act == 1, "act_mul: unknown activation %d", act);
-  const size_t total = (size_t)T * I;
-  const int blocks = (int)((total + 255) / 256 > 65535 * 4 ? 65535 * 4 : (total + 255) / 256);
-  hipStream_t s = (hipStream_t)stream;
-  if (dtype == NHV_F32)
-    hipLaunchKernelGGL(act_mul_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gu, (float*)out, I, total, act);
-  else if (dtype == NHV_BF16)
-    hipLaunchKernelGGL(act_mul_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)out, I, total, act);
-  else
-    return nhv_fail("act_mul: unknown dtype %d", dtype);
-  NHV_LAUNCH_CHECK("act_mul");
   return 0;
 }

@@ -188,9 +188,10 @@ extern "C" int nhv_experts_down(const void* u, const void* ids, const void* down
 // ---------------------------------------------------------------- many rows in bfloat16: the pairs sorted by expert
 // The (token, expert) pairs of a step are put in the order of their experts, every expert's run filled up to whole
 // tiles of TM pairs (-1 where there is none), so that a block meets one expert's matrices only: nhv_experts_sort.
-// nhv_experts_grouped_gate_up and nhv_experts_grouped_down are then matrix products on the matrix cores in which a
-// block owns one tile of pairs and some tiles of 16 outputs; its waves share the inner dimension and their sums meet
-// in LDS in the order of the waves. A pair's sums do not depend on where the sort has put it.
+// nhv_experts_grouped_gate_up and nhv_experts_grouped_down are then matrix products on the matrix cores. With tiles of
+// 16 pairs (few pairs an expert) a block owns one tile of pairs and some tiles of 16 outputs; its waves share the
+// inner dimension and their sums meet in LDS in the order of the waves. With tiles of 64 pairs the block's pieces of
+// both operands go through LDS (experts_tiled_kernel). A pair's sums do not depend on where the sort has put it.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
@@ -349,6 +350,118 @@ __global__ __launch_bounds__(64 * WAVES) void experts_grouped_kernel(const bf16_
   }
 }
 
+// Tiles of 64 pairs (BM; the kernel is written for any multiple of 16 a wave row): a block of WM x WN waves owns BM pairs x BW rows of the expert's matrix (GLU: BW / 2 gate
+// rows and their up rows, so BW / 2 outputs; else BW outputs) and walks over k in pieces of 64 that all its threads
+// bring into LDS (the next piece is asked for, into registers, while this one is computed). A wave takes BM / 16 / WM
+// tiles of pairs against BW / 16 / WN tiles of matrix rows (GLU: gate tiles and their up tiles). The larger the block's
+// tile, the fewer bytes cross from L2 for a product: 64 x 128 asks for 24 KB per 2^20 multiply-adds, 128 x 256 for 48 KB
+// per 2^22.
+template <bool GLU, typename TOut, int BM, int BW, int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN) void experts_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                                     TOut* __restrict__ y, const int* __restrict__ sorted,
+                                                                     const int* __restrict__ tile_expert,
+                                                                     const float* __restrict__ scores, int top, int N, int K,
+                                                                     int act) {
+  constexpr int THREADS = 64 * WM * WN, BK = 64, LD = BK + 8;  // (rows of 144 bytes: 16-byte pieces stay aligned, banks shift)
+  constexpr int RP = THREADS / 8;            // rows that the threads bring in one pass
+  constexpr int XI = BM / RP, WI = BW / RP;
+  constexpr int MT = BM / 16 / WM, NT = BW / 16 / WN, NH = GLU ? NT / 2 : NT;
+  constexpr int OUT = GLU ? BW / 2 : BW;     // outputs a block
+  static_assert(XI >= 1 && WI >= 1 && MT >= 1 && NH >= 1, "tile sizes and waves do not fit");
+  __shared__ __attribute__((aligned(16))) bf16_t xs[BM * LD];
+  __shared__ __attribute__((aligned(16))) bf16_t ws[BW * LD];
+  const int e = tile_expert[blockIdx.x];
+  if (e < 0) return;                         // the same for the whole block
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, grp = lane >> 4;
+  const int wm = wave / WN, wn = wave % WN;
+  const int* places = sorted + (size_t)blockIdx.x * BM;
+  const int n0 = blockIdx.y * OUT;
+  const bf16_t* wbase = w + (size_t)e * (GLU ? 2 : 1) * N * K;
+  // what this thread brings: 8 entries at k offset kc of rows r0 + RP i of x and of the matrix piece
+  const int kc = (tid & 7) * 8, r0 = tid >> 3;
+  const bf16_t* xp[XI];
+  bool xok[XI];
+#pragma unroll
+  for (int i = 0; i < XI; ++i) {
+    const int pair = places[r0 + RP * i];
+    xok[i] = pair >= 0;
+    xp[i] = x + (size_t)(xok[i] ? (GLU ? pair / top : pair) : 0) * K + kc;
+  }
+  const bf16_t* wp[WI];
+  bool wok[WI];
+#pragma unroll
+  for (int i = 0; i < WI; ++i) {
+    const int r = r0 + RP * i;
+    const int n = GLU ? n0 + r % OUT : n0 + r;
+    wok[i] = n < N;
+    const size_t row = GLU ? (size_t)(r / OUT) * N + n : (size_t)n;
+    wp[i] = wbase + (wok[i] ? row : 0) * K + kc;
+  }
+  bf16x8 xr[XI], wr[WI];
+  auto ask = [&](int k0) {
+    const bool k_ok = k0 + kc < K;
+#pragma unroll
+    for (int i = 0; i < XI; ++i) xr[i] = (xok[i] && k_ok) ? ex_load8(xp[i] + k0) : ex_zero8();
+#pragma unroll
+    for (int i = 0; i < WI; ++i) wr[i] = (wok[i] && k_ok) ? ex_load8(wp[i] + k0) : ex_zero8();
+  };
+  floatx4 acc[NT][MT];
+#pragma unroll
+  for (int a = 0; a < NT; ++a)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[a][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // the rows of the matrix piece that this wave's tile a starts at: GLU: gate tiles first, then their up tiles
+  auto tile_row = [&](int a) { return GLU ? (a / NH) * OUT + (wn * NH + a % NH) * 16 : (wn * NT + a) * 16; };
+  ask(0);
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    __syncthreads();                         // the piece before is computed
+#pragma unroll
+    for (int i = 0; i < XI; ++i) *reinterpret_cast<bf16x8*>(&xs[(r0 + RP * i) * LD + kc]) = xr[i];
+#pragma unroll
+    for (int i = 0; i < WI; ++i) *reinterpret_cast<bf16x8*>(&ws[(r0 + RP * i) * LD + kc]) = wr[i];
+    __syncthreads();
+    if (k0 + BK < K) ask(k0 + BK);
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 32) {
+      bf16x8 b[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        b[mt] = *reinterpret_cast<const bf16x8*>(&xs[((wm * MT + mt) * 16 + col) * LD + kk + grp * 8]);
+#pragma unroll
+      for (int a = 0; a < NT; ++a) {
+        const bf16x8 af = *reinterpret_cast<const bf16x8*>(&ws[(tile_row(a) + col) * LD + kk + grp * 8]);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, b[mt], acc[a][mt], 0, 0, 0);
+      }
+    }
+  }
+  // a lane holds, of every tile, four outputs (grp * 4 + j) of the pair at place (wm MT + mt) * 16 + col
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int pair = places[(wm * MT + mt) * 16 + col];
+    if (pair < 0) continue;
+    const float s = GLU ? scores[pair] : 1.0f;
+#pragma unroll
+    for (int a = 0; a < NH; ++a)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + (wn * NH + a) * 16 + grp * 4 + j;
+        if (n >= N) continue;
+        if (GLU) y[(size_t)pair * N + n] = (TOut)(nhv_expert_act(s * acc[a][mt][j], act) * (s * acc[NH + a][mt][j]));
+        else y[(size_t)pair * N + n] = (TOut)acc[a][mt][j];
+      }
+  }
+}
+
+template <bool GLU, typename TOut>
+static void tiled_launch(hipStream_t s, const void* x, const void* w, void* y, const void* sorted, const void* tile_expert,
+                         const void* scores, int top, int N, int K, int act, int tiles_cap) {
+  const int out = GLU ? 64 : 128;
+  hipLaunchKernelGGL((experts_tiled_kernel<GLU, TOut, 64, 128, 1, 4>), dim3(tiles_cap, (N + out - 1) / out), dim3(256), 0, s,
+                     (const bf16_t*)x, (const bf16_t*)w, (TOut*)y, (const int*)sorted, (const int*)tile_expert,
+                     (const float*)scores, top, N, K, act);
+}
+
 template <int MT, bool GLU, typename TOut>
 static void grouped_launch(hipStream_t s, const void* x, const void* w, void* y, const void* sorted, const void* tile_expert,
                            const void* scores, int top, int N, int K, int act, int tiles_cap) {
@@ -367,7 +480,7 @@ extern "C" int nhv_experts_grouped_gate_up(const void* h, const void* gate_up, v
               "experts_grouped_gate_up: bad sizes W=%d (a multiple of 8) F=%d top=%d TM=%d", W, F, top, TM);
   NHV_REQUIRE((F + 31) / 32 <= 65535, "experts_grouped_gate_up: F=%d is beyond this kernel's grid", F);
   hipStream_t s = (hipStream_t)stream;
-  if (TM == 64) grouped_launch<4, true, bf16_t>(s, h, gate_up, u, sorted, tile_expert, scores, top, F, W, act, tiles_cap);
+  if (TM >= 64) tiled_launch<true, bf16_t>(s, h, gate_up, u, sorted, tile_expert, scores, top, F, W, act, tiles_cap);
   else grouped_launch<1, true, bf16_t>(s, h, gate_up, u, sorted, tile_expert, scores, top, F, W, act, tiles_cap);
   NHV_LAUNCH_CHECK("experts_grouped_gate_up");
   return 0;
@@ -380,7 +493,7 @@ extern "C" int nhv_experts_grouped_down(const void* u, const void* down, void* y
               "experts_grouped_down: bad sizes W=%d F=%d (a multiple of 8) TM=%d", W, F, TM);
   NHV_REQUIRE((W + 63) / 64 <= 65535, "experts_grouped_down: W=%d is beyond this kernel's grid", W);
   hipStream_t s = (hipStream_t)stream;
-  if (TM == 64) grouped_launch<4, false, float>(s, u, down, y, sorted, tile_expert, nullptr, 1, W, F, 0, tiles_cap);
+  if (TM >= 64) tiled_launch<false, float>(s, u, down, y, sorted, tile_expert, nullptr, 1, W, F, 0, tiles_cap);
   else grouped_launch<1, false, float>(s, u, down, y, sorted, tile_expert, nullptr, 1, W, F, 0, tiles_cap);
   NHV_LAUNCH_CHECK("experts_grouped_down");
   return 0;

@@ -264,7 +264,7 @@ class NativeBackend:
 
     def act_mul(self, gu, out, act):
         T, I = out.shape
-        self._call("nhv_act_mul", _ptr(gu), _ptr(out), T, I, act, dtype_code(gu), _stream())
+        self._call("nhv_gelu_tanh_mul" if act == 1 else "nhv_silu_mul", _ptr(gu), _ptr(out), T, I, dtype_code(gu), _stream())
 
     # -- attention over a cached latent --
     def latent_prepare(self, a, q_off, q_rank, c_off, kv_rank, rot, wq, wc, eps, freqs, gain, positions, slot_mapping,
@@ -283,18 +283,20 @@ class NativeBackend:
         gate_p = None if gate is None else ctypes.c_void_p(gate.data_ptr() + 4 * gate_off)
         x_p, y_p = ctypes.c_void_p(x.data_ptr() + item * x_off), ctypes.c_void_p(y.data_ptr() + item * y_off)
         gs_t = LL(0 if gate is None else gate.shape[1])
-        if T <= 16 and K <= 1024:
+        if T <= 16 and 16 * K * 4 + (64 * item + 4) * K <= 96 * 1024:      # (the kernel keeps the rows and a piece of the matrix in LDS)
             rot, xr, yr, freqs, gain, positions = turn if turn is not None else (0, 0, 0, None, 1.0, None)
             self._call("nhv_head_gemm_fewrows", x_p, LL(H * x_row), LL(x_row), _ptr(w), LL(w_head), LL(w_n), LL(w_k), y_p,
                        LL(H * y_row), LL(y_row), gate_p, gs_t, T, H, N, K, rot, xr - x_off, yr - y_off, _ptr(freqs),
                        ctypes.c_float(gain), _ptr(positions), dtype_code(x), _stream())
             return True
-        if x.dtype == torch.bfloat16 and not self.own_kernels_only and gate is None:
+        if x.dtype == torch.bfloat16 and not self.own_kernels_only and (gate is None or (y_off == 0 and y_row == N)):
             # many rows: the library's batched product, one matrix per head, on strided views
             xv = x[:, :, x_off:x_off + K].transpose(0, 1)                         # [H, T, K]
             wv = torch.as_strided(w, (H, K, N), (w_head, w_k, w_n))
             yv = y[:, :, y_off:y_off + N].transpose(0, 1)
             yv.copy_(torch.bmm(xv, wv))
+            if gate is not None:
+                self._call("nhv_head_gate", _ptr(y), gate_p, gs_t, T, H, N, dtype_code(y), _stream())
             return False
         self._call("nhv_head_gemm", x_p, LL(H * x_row), LL(x_row), _ptr(w), LL(w_head), LL(w_n), LL(w_k), y_p, LL(H * y_row),
                    LL(y_row), gate_p, gs_t, T, H, N, K, dtype_code(x), _stream())
@@ -323,7 +325,10 @@ class NativeBackend:
         E, F2, _ = gate_up.shape
         F, top = F2 // 2, ids.shape[1]
         P = T * top
-        TM = 64 if P >= 32 * E else 16                  # places a tile: runs of an expert's pairs are filled up to whole tiles
+        # places a tile (runs of an expert's pairs are filled up to whole tiles): 64 where an expert has pairs enough.
+        # (Tiles of 128 pairs x 256 matrix rows, which the kernel can be built for as well, took the same time at 4,096
+        # pairs of 16 experts: half the bytes from L2, but one block a compute unit, which then waits for every piece.)
+        TM = 64 if P >= 32 * E else 16
         tiles = -(-P // TM) + E
         index = torch.empty(tiles * TM + tiles, dtype=torch.int32, device=h.device)
         sorted_pairs, tile_expert = index[:tiles * TM], index[tiles * TM:]

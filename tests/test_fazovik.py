@@ -242,7 +242,7 @@ def test_routed_experts_alone(where, kernels):
     dt = _dt(dtype)
     g = torch.Generator().manual_seed(8)
     for E, top, F, W, T in ((5, 2, 12, 20, 9), (1, 1, 8, 16, 3), (7, 7, 4, 12, 4), (70, 3, 8, 24, 21), (2, 1, 16, 32, 70),
-                            (3, 2, 24, 40, 130)):
+                            (3, 2, 24, 40, 130), (2, 2, 136, 72, 300)):
         w = {"router": (torch.randn(E, W, generator=g) * 0.6).to(torch.bfloat16).double()}
         for e in range(E):
             w[f"e{e}.gate"] = (torch.randn(F, W, generator=g) / W ** 0.5).to(torch.bfloat16).double()
