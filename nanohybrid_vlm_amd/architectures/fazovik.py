@@ -289,7 +289,9 @@ def _shape(layers: int, width: int, vocab: int, heads: int, dim: int, rot_dim: i
 SHAPES = {
     "fazovik-tiny": _shape(8, 64, 197, 3, 16, 8, 16, 24, 24, 96, 4, 2, 32, 61),
     "fazovik-1b": _shape(16, 2048, 32768, 16, 128, 64, 128, 768, 192, 6144, 16, 2, 1536, 65521),
-    "fazovik-8b": _shape(36, 4096, 151936, 32, 128, 64, 128, 1536, 448, 12288, 32, 4, 1536, 262139),
+    "fazovik-8b": _shape(36, 4096, 151936, 32, 128, 64, 128, 1536, 192, 12288, 32, 4, 1536, 262139),
+    # stored rows of 512 entries: more than the matrix-core attention kernels take (256), so attention is the plain kernel's
+    "fazovik-8b-wide": _shape(36, 4096, 151936, 32, 128, 64, 128, 1536, 448, 12288, 32, 4, 1536, 262139),
 }
 
 

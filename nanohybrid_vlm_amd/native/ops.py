@@ -186,6 +186,13 @@ class NativeBackend:
             window = -chunk
         if fast and batch.max_q_len == 1 and Hq // Hkv <= 16 and T <= 65535:
             return self._decode_attention(q, k_cache, v_cache, out, batch, block_tables, scale, window)
+        if fast and batch.max_q_len == 1 and Hkv == 1 and T <= 65535:
+            # more than 16 query heads on one key/value head (a cached latent): sixteen heads at a time
+            for h0 in range(0, Hq, 16):
+                part = torch.empty((T, min(16, Hq - h0), E), dtype=out.dtype, device=out.device)
+                self._decode_attention(q[:, h0:h0 + 16].contiguous(), k_cache, v_cache, part, batch, block_tables, scale, window)
+                out[:, h0:h0 + 16] = part
+            return None
         if fast and batch.num_requests <= 65535 and Hkv <= 65535:
             # prompt portions (and whatever single tokens share their batch) on the matrix cores
             return self._call("nhv_prefill_attention_bf16", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out),
