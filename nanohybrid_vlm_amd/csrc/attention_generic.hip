@@ -11,7 +11,7 @@
 #include "nhv_common.h"
 #include <math.h>
 
-#define MAX_D_CHUNKS 8   // head sizes up to 512
+#define MAX_D_CHUNKS 16  // head sizes up to 1024 (a cached latent's rows are longer than ordinary heads)
 
 template <typename T>
 __global__ __launch_bounds__(256) void paged_attention_generic_kernel(

@@ -168,7 +168,24 @@ extern "C" int nhv_head_gemm(const void* x, long long xs_t, long long xs_h, cons
 // of the rows, k rising as above, so the sums are the same bits. One more block a head may turn the rotated part of x
 // and copy it beside the outputs (``rot`` entries from x_rot_off to y_rot_off), which saves the launch of
 // nhv_rotate_interleaved.
-template <typename T>
+template <typename V>
+__device__ __forceinline__ void hg_load8f(const V* p, float* out);
+template <>
+__device__ __forceinline__ void hg_load8f<bf16_t>(const bf16_t* p, float* out) {
+  typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 v8;
+  const v8 v = *reinterpret_cast<const v8*>(p);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = (float)v[e];
+}
+template <>
+__device__ __forceinline__ void hg_load8f<float>(const float* p, float* out) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w; out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+}
+
+// VEC: K and N are multiples of 8 and every row of x and of the matrix starts at a multiple of 8 entries from an
+// address that is a multiple of 32 bytes (the host checks), so eight entries can be asked for at once.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void head_gemm_fewrows_kernel(const T* __restrict__ x, long long xs_t, long long xs_h,
                                                                 const T* __restrict__ w, long long ws_h, long long ws_n,
                                                                 long long ws_k, T* __restrict__ y, long long ys_t,
@@ -191,26 +208,72 @@ __global__ __launch_bounds__(256) void head_gemm_fewrows_kernel(const T* __restr
     }
     return;
   }
-  // [K][LDW]: rows one bank longer than 64 outputs, so that threads that walk along k (a matrix that is contiguous in k)
-  // store into different banks
-  constexpr int LDW = 64 + 4 / (int)sizeof(T);
+  // [K][LDW]: rows a little longer than 64 outputs: pieces of 16 bytes stay aligned, and threads that walk along k (a
+  // matrix that is contiguous in k) do not all store into one bank
+  constexpr int LDW = 64 + 16 / (int)sizeof(T);
   T* wl = reinterpret_cast<T*>(xs + 16 * K);
   const int n0 = blockIdx.x * 64;
   const T* wh = w + (size_t)h * ws_h;
-  if (ws_k == 1) {                           // a row of the matrix is contiguous in k: threads walk along k
-    for (int i = threadIdx.x; i < 64 * K; i += blockDim.x) {
-      const int n = i / K, k = i % K;
-      wl[k * LDW + n] = n0 + n < N ? wh[(size_t)(n0 + n) * ws_n + k] : from_f32<T>(0.f);
+  const T* xh = x + (size_t)h * xs_h;
+  if (VEC) {
+    // eight entries a load, and all of a thread's loads asked for before the first is stored (the matrix comes from
+    // memory: a thread that stored each piece before it asked for the next waited once a piece)
+    const int w_chunks = 8 * K;              // 64 x K / 8
+    for (int c0 = 0; c0 < w_chunks; c0 += 256 * 8) {
+      float v[8][8];
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const int c = c0 + b * 256 + (int)threadIdx.x;
+        if (c >= w_chunks) continue;
+        int n, k;
+        if (ws_k == 1) { n = c / (K / 8); k = (c % (K / 8)) * 8; }
+        else { k = c / 8; n = (c % 8) * 8; }
+        const bool ok = ws_k == 1 ? n0 + n < N : n0 + n + 7 < N;
+        if (ok) hg_load8f(wh + (size_t)(n0 + n) * ws_n + (size_t)k * ws_k, v[b]);
+        else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) v[b][i] = (ws_k != 1 && n0 + n + i < N) ? to_f32(wh[(size_t)(n0 + n + i) + (size_t)k * ws_k]) : 0.f;
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const int c = c0 + b * 256 + (int)threadIdx.x;
+        if (c >= w_chunks) continue;
+        if (ws_k == 1) {
+          const int n = c / (K / 8), k = (c % (K / 8)) * 8;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) wl[(k + i) * LDW + n] = from_f32<T>(v[b][i]);
+        } else {
+          const int k = c / 8, n = (c % 8) * 8;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) wl[k * LDW + n + i] = from_f32<T>(v[b][i]);
+        }
+      }
     }
-  } else {                                   // contiguous in n
-    for (int i = threadIdx.x; i < 64 * K; i += blockDim.x) {
-      const int k = i / 64, n = i % 64;
-      wl[k * LDW + n] = n0 + n < N ? wh[(size_t)(n0 + n) * ws_n + (size_t)k * ws_k] : from_f32<T>(0.f);
+    const int x_chunks = 2 * K;              // 16 x K / 8
+    for (int c = threadIdx.x; c < x_chunks; c += blockDim.x) {
+      const int t = c / (K / 8), k = (c % (K / 8)) * 8;
+      float v[8];
+      if (t < rows) hg_load8f(xh + (size_t)t * xs_t + k, v);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xs[t * K + k + i] = t < rows ? v[i] : 0.f;
     }
-  }
-  for (int i = threadIdx.x; i < 16 * K; i += blockDim.x) {
-    const int t = i / K, k = i % K;
-    xs[i] = t < rows ? to_f32(x[(size_t)t * xs_t + (size_t)h * xs_h + k]) : 0.f;
+  } else {
+    if (ws_k == 1) {                         // a row of the matrix is contiguous in k: threads walk along k
+      for (int i = threadIdx.x; i < 64 * K; i += blockDim.x) {
+        const int n = i / K, k = i % K;
+        wl[k * LDW + n] = n0 + n < N ? wh[(size_t)(n0 + n) * ws_n + k] : from_f32<T>(0.f);
+      }
+    } else {                                 // contiguous in n
+      for (int i = threadIdx.x; i < 64 * K; i += blockDim.x) {
+        const int k = i / 64, n = i % 64;
+        wl[k * LDW + n] = n0 + n < N ? wh[(size_t)(n0 + n) * ws_n + (size_t)k * ws_k] : from_f32<T>(0.f);
+      }
+    }
+    for (int i = threadIdx.x; i < 16 * K; i += blockDim.x) {
+      const int t = i / K, k = i % K;
+      xs[i] = t < rows ? to_f32(xh[(size_t)t * xs_t + k]) : 0.f;
+    }
   }
   __syncthreads();
   const int lane = threadIdx.x & 63, t0 = (threadIdx.x >> 6) * 4;
@@ -237,7 +300,7 @@ extern "C" int nhv_head_gemm_fewrows(const void* x, long long xs_t, long long xs
                                      long long gs_t, int rows, int H, int N, int K, int rot, int x_rot_off, int y_rot_off,
                                      const void* freqs, float gain, const void* positions, int dtype, void* stream) {
   const size_t item = dtype == NHV_F32 ? 4 : 2;
-  const size_t lds = 16 * (size_t)K * sizeof(float) + (64 + 4 / item) * (size_t)K * item;
+  const size_t lds = 16 * (size_t)K * sizeof(float) + (64 + 16 / item) * (size_t)K * item;
   NHV_REQUIRE(rows > 0 && rows <= 16 && H > 0 && H <= 65535 && N > 0 && K > 0 && lds <= 96 * 1024,
               "head_gemm_fewrows: bad sizes rows=%d (up to 16) H=%d N=%d K=%d (LDS of %zu bytes, up to 98304)", rows, H, N, K, lds);
   NHV_REQUIRE(rot >= 0 && rot % 2 == 0 && (rot == 0 || (freqs != nullptr && positions != nullptr)),
@@ -245,19 +308,25 @@ extern "C" int nhv_head_gemm_fewrows(const void* x, long long xs_t, long long xs
   const int n_chunks = (N + 63) / 64;
   const dim3 grid(n_chunks + (rot > 0 ? 1 : 0), H);
   hipStream_t s = (hipStream_t)stream;
+  const long long strides[] = {xs_t, xs_h, ws_h, ws_n == 1 ? ws_k : ws_n};
+  bool vec = K % 8 == 0 && N % 8 == 0 && (uintptr_t)x % 32 == 0 && (uintptr_t)w % 32 == 0 && (ws_n == 1 || ws_k == 1);
+  for (long long st : strides) vec = vec && st % 8 == 0;
+#define NHV_HG_LAUNCH(TYPE, VEC)                                                                                          \
+  do {                                                                                                                    \
+    if (lds > 64 * 1024)                                                                                                  \
+      (void)hipFuncSetAttribute((const void*)head_gemm_fewrows_kernel<TYPE, VEC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+    hipLaunchKernelGGL((head_gemm_fewrows_kernel<TYPE, VEC>), grid, dim3(256), lds, s, (const TYPE*)x, xs_t, xs_h,          \
+                       (const TYPE*)w, ws_h, ws_n, ws_k, (TYPE*)y, ys_t, ys_h, (const float*)gate, gs_t, rows, N, K, n_chunks, \
+                       rot, x_rot_off, y_rot_off, (const double*)freqs, gain, (const int*)positions);                      \
+  } while (0)
   if (dtype == NHV_F32) {
-    if (lds > 64 * 1024) hipFuncSetAttribute((const void*)head_gemm_fewrows_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(head_gemm_fewrows_kernel<float>, grid, dim3(256), lds, s, (const float*)x, xs_t, xs_h, (const float*)w,
-                       ws_h, ws_n, ws_k, (float*)y, ys_t, ys_h, (const float*)gate, gs_t, rows, N, K, n_chunks, rot, x_rot_off,
-                       y_rot_off, (const double*)freqs, gain, (const int*)positions);
+    if (vec) NHV_HG_LAUNCH(float, true); else NHV_HG_LAUNCH(float, false);
   } else if (dtype == NHV_BF16) {
-    if (lds > 64 * 1024) hipFuncSetAttribute((const void*)head_gemm_fewrows_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(head_gemm_fewrows_kernel<bf16_t>, grid, dim3(256), lds, s, (const bf16_t*)x, xs_t, xs_h,
-                       (const bf16_t*)w, ws_h, ws_n, ws_k, (bf16_t*)y, ys_t, ys_h, (const float*)gate, gs_t, rows, N, K,
-                       n_chunks, rot, x_rot_off, y_rot_off, (const double*)freqs, gain, (const int*)positions);
+    if (vec) NHV_HG_LAUNCH(bf16_t, true); else NHV_HG_LAUNCH(bf16_t, false);
   } else {
     return nhv_fail("head_gemm_fewrows: unknown dtype %d", dtype);
   }
+#undef NHV_HG_LAUNCH
   NHV_LAUNCH_CHECK("head_gemm_fewrows");
   return 0;
 }

@@ -290,7 +290,7 @@ class NativeBackend:
         gate_p = None if gate is None else ctypes.c_void_p(gate.data_ptr() + 4 * gate_off)
         x_p, y_p = ctypes.c_void_p(x.data_ptr() + item * x_off), ctypes.c_void_p(y.data_ptr() + item * y_off)
         gs_t = LL(0 if gate is None else gate.shape[1])
-        if T <= 16 and 16 * K * 4 + (64 * item + 4) * K <= 96 * 1024:      # (the kernel keeps the rows and a piece of the matrix in LDS)
+        if T <= 16 and 16 * K * 4 + (64 * item + 16) * K <= 96 * 1024:      # (the kernel keeps the rows and a piece of the matrix in LDS)
             rot, xr, yr, freqs, gain, positions = turn if turn is not None else (0, 0, 0, None, 1.0, None)
             self._call("nhv_head_gemm_fewrows", x_p, LL(H * x_row), LL(x_row), _ptr(w), LL(w_head), LL(w_n), LL(w_k), y_p,
                        LL(H * y_row), LL(y_row), gate_p, gs_t, T, H, N, K, rot, xr - x_off, yr - y_off, _ptr(freqs),
