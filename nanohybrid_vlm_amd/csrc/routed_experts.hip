@@ -190,7 +190,7 @@ extern "C" int nhv_experts_down(const void* u, const void* ids, const void* down
 // tiles of TM pairs (-1 where there is none), so that a block meets one expert's matrices only: nhv_experts_sort.
 // nhv_experts_grouped_gate_up and nhv_experts_grouped_down are then matrix products on the matrix cores. With tiles of
 // 16 pairs (few pairs an expert) a block owns one tile of pairs and some tiles of 16 outputs; its waves share the
-// inner dimension and their sums meet in LDS in the order of the waves. With tiles of 64 pairs the block's pieces of
+// inner dimension and their sums meet in LDS in the order of the waves. With tiles of 64 or 128 pairs the block's pieces of
 // both operands go through LDS (experts_tiled_kernel). A pair's sums do not depend on where the sort has put it.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(64 * WAVES) void experts_grouped_kernel(const bf16_
   }
 }
 
-// Tiles of 64 pairs (BM; the kernel is written for any multiple of 16 a wave row): a block of WM x WN waves owns BM pairs x BW rows of the expert's matrix (GLU: BW / 2 gate
+// Tiles of 64 or 128 pairs (BM): a block of WM x WN waves owns BM pairs x BW rows of the expert's matrix (GLU: BW / 2 gate
 // rows and their up rows, so BW / 2 outputs; else BW outputs) and walks over k in pieces of 64 that all its threads
 // bring into LDS (the next piece is asked for, into registers, while this one is computed). A wave takes BM / 16 / WM
 // tiles of pairs against BW / 16 / WN tiles of matrix rows (GLU: gate tiles and their up tiles). The larger the block's
@@ -455,11 +455,15 @@ __global__ __launch_bounds__(64 * WM * WN) void experts_tiled_kernel(const bf16_
 
 template <bool GLU, typename TOut>
 static void tiled_launch(hipStream_t s, const void* x, const void* w, void* y, const void* sorted, const void* tile_expert,
-                         const void* scores, int top, int N, int K, int act, int tiles_cap) {
+                         const void* scores, int top, int N, int K, int act, int tiles_cap, int TM) {
   const int out = GLU ? 64 : 128;
-  hipLaunchKernelGGL((experts_tiled_kernel<GLU, TOut, 64, 128, 1, 4>), dim3(tiles_cap, (N + out - 1) / out), dim3(256), 0, s,
-                     (const bf16_t*)x, (const bf16_t*)w, (TOut*)y, (const int*)sorted, (const int*)tile_expert,
-                     (const float*)scores, top, N, K, act);
+  const dim3 grid(tiles_cap, (N + out - 1) / out);
+  if (TM == 128)
+    hipLaunchKernelGGL((experts_tiled_kernel<GLU, TOut, 128, 128, 2, 4>), grid, dim3(512), 0, s, (const bf16_t*)x,
+                       (const bf16_t*)w, (TOut*)y, (const int*)sorted, (const int*)tile_expert, (const float*)scores, top, N, K, act);
+  else
+    hipLaunchKernelGGL((experts_tiled_kernel<GLU, TOut, 64, 128, 1, 4>), grid, dim3(256), 0, s, (const bf16_t*)x,
+                       (const bf16_t*)w, (TOut*)y, (const int*)sorted, (const int*)tile_expert, (const float*)scores, top, N, K, act);
 }
 
 template <int MT, bool GLU, typename TOut>
@@ -472,15 +476,15 @@ static void grouped_launch(hipStream_t s, const void* x, const void* w, void* y,
                      (const float*)scores, top, N, K, act);
 }
 
-// u [pairs, F] bfloat16 from the step's rows h [tokens, W]; TM: 16 or 64 places a tile (as the sort was told).
+// u [pairs, F] bfloat16 from the step's rows h [tokens, W]; TM: 16, 64 or 128 places a tile (as the sort was told).
 extern "C" int nhv_experts_grouped_gate_up(const void* h, const void* gate_up, void* u, const void* sorted,
                                            const void* tile_expert, const void* scores, int top, int W, int F, int act,
                                            int TM, int tiles_cap, void* stream) {
-  NHV_REQUIRE(W > 0 && F > 0 && W % 8 == 0 && top > 0 && tiles_cap > 0 && (TM == 16 || TM == 64),
+  NHV_REQUIRE(W > 0 && F > 0 && W % 8 == 0 && top > 0 && tiles_cap > 0 && (TM == 16 || TM == 64 || TM == 128),
               "experts_grouped_gate_up: bad sizes W=%d (a multiple of 8) F=%d top=%d TM=%d", W, F, top, TM);
   NHV_REQUIRE((F + 31) / 32 <= 65535, "experts_grouped_gate_up: F=%d is beyond this kernel's grid", F);
   hipStream_t s = (hipStream_t)stream;
-  if (TM >= 64) tiled_launch<true, bf16_t>(s, h, gate_up, u, sorted, tile_expert, scores, top, F, W, act, tiles_cap);
+  if (TM >= 64) tiled_launch<true, bf16_t>(s, h, gate_up, u, sorted, tile_expert, scores, top, F, W, act, tiles_cap, TM);
   else grouped_launch<1, true, bf16_t>(s, h, gate_up, u, sorted, tile_expert, scores, top, F, W, act, tiles_cap);
   NHV_LAUNCH_CHECK("experts_grouped_gate_up");
   return 0;
@@ -489,11 +493,11 @@ extern "C" int nhv_experts_grouped_gate_up(const void* h, const void* gate_up, v
 // y [pairs, W] float from u [pairs, F] bfloat16.
 extern "C" int nhv_experts_grouped_down(const void* u, const void* down, void* y, const void* sorted,
                                         const void* tile_expert, int W, int F, int TM, int tiles_cap, void* stream) {
-  NHV_REQUIRE(W > 0 && F > 0 && F % 8 == 0 && tiles_cap > 0 && (TM == 16 || TM == 64),
+  NHV_REQUIRE(W > 0 && F > 0 && F % 8 == 0 && tiles_cap > 0 && (TM == 16 || TM == 64 || TM == 128),
               "experts_grouped_down: bad sizes W=%d F=%d (a multiple of 8) TM=%d", W, F, TM);
   NHV_REQUIRE((W + 63) / 64 <= 65535, "experts_grouped_down: W=%d is beyond this kernel's grid", W);
   hipStream_t s = (hipStream_t)stream;
-  if (TM >= 64) tiled_launch<false, float>(s, u, down, y, sorted, tile_expert, nullptr, 1, W, F, 0, tiles_cap);
+  if (TM >= 64) tiled_launch<false, float>(s, u, down, y, sorted, tile_expert, nullptr, 1, W, F, 0, tiles_cap, TM);
   else grouped_launch<1, false, float>(s, u, down, y, sorted, tile_expert, nullptr, 1, W, F, 0, tiles_cap);
   NHV_LAUNCH_CHECK("experts_grouped_down");
   return 0;

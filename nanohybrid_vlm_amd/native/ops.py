@@ -332,10 +332,11 @@ class NativeBackend:
         E, F2, _ = gate_up.shape
         F, top = F2 // 2, ids.shape[1]
         P = T * top
-        # places a tile (runs of an expert's pairs are filled up to whole tiles): 64 where an expert has pairs enough.
-        # (Tiles of 128 pairs x 256 matrix rows, which the kernel can be built for as well, took the same time at 4,096
-        # pairs of 16 experts: half the bytes from L2, but one block a compute unit, which then waits for every piece.)
-        TM = 64 if P >= 32 * E else 16
+        # places a tile (runs of an expert's pairs are filled up to whole tiles): 128 or 64 where an expert has pairs
+        # enough (block tiles of 128 x 128 and 64 x 128 matrix rows). Tiles of 128 pairs x 256 matrix rows, which the
+        # kernel can be built for as well, took the time of 64 x 128 at 4,096 pairs of 16 experts: half the bytes from
+        # L2, but one block a compute unit, which then waits for every piece; 128 x 128 takes a tenth less.
+        TM = 128 if P >= 192 * E else (64 if P >= 32 * E else 16)
         tiles = -(-P // TM) + E
         index = torch.empty(tiles * TM + tiles, dtype=torch.int32, device=h.device)
         sorted_pairs, tile_expert = index[:tiles * TM], index[tiles * TM:]
