@@ -218,7 +218,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_kernel(const bf16_t* 
     const int n = n0 + nt * 16 + grp * 4 + j;           // the tile's row 4 grp + j is output n, its column is row col of x
     float r = v[0][j] * rs;
     if (bias && n < N) r += (float)bias[n];
-    if (GLU) r = r / (1.0f + expf(-r)) * (v[NA - 1][j] * rs);
+    if (GLU) r = nhv_glu_gate(r, f.glu_act) * (v[NA - 1][j] * rs);
     out[j] = r;
   }
   emit_tile<FUSED, TOut>(f, out, y, col, grp, n0 + nt * 16, blockIdx.x * NT + nt, (N + 15) / 16, M, N);
@@ -344,7 +344,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_resident_kernel(const
       const int n = n0 + grp * 4 + j;
       float r = v[0][j] * rs;
       if (bias && n < N) r += (float)bias[n];
-      if (GLU) r = r / (1.0f + expf(-r)) * (v[NA - 1][j] * rs);
+      if (GLU) r = nhv_glu_gate(r, f.glu_act) * (v[NA - 1][j] * rs);
       out[j] = r;
     }
     emit_tile<FUSED && !GLU, TOut>(f, out, y, col, grp, n0, tile, tiles, M, N, res_ahead);
@@ -448,7 +448,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_pieces_kernel(const b
       const int n = n0 + grp * 4 + j;
       float r = v[0][j] * rs;
       if (bias && n < N) r += (float)bias[n];
-      if (GLU) r = r / (1.0f + expf(-r)) * (v[NA - 1][j] * rs);
+      if (GLU) r = nhv_glu_gate(r, f.glu_act) * (v[NA - 1][j] * rs);
       out[j] = r;
     }
     emit_tile<FUSED, TOut>(f, out, y, col, grp, n0, tile, tiles, M, N);
@@ -560,7 +560,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_fewrows_passes_kernel(const b
         const int n = n0 + grp * 4 + j;
         float r = v[0][j] * rs;
         if (bias && n < N) r += (float)bias[n];
-        if (GLU) r = r / (1.0f + expf(-r)) * (v[NA - 1][j] * rs);
+        if (GLU) r = nhv_glu_gate(r, f.glu_act) * (v[NA - 1][j] * rs);
         out[j] = r;
       }
       emit_tile<FUSED, TOut>(f, out, y, col, grp, n0, tile, tiles, M, N);

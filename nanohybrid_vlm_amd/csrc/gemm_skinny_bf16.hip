@@ -180,6 +180,18 @@ extern "C" int nhv_gemm_skinny_glu_bf16(const void* x, const void* w, void* y, i
   return 0;
 }
 
+// The same for up to 16 rows with the gate's activation named: 0 SiLU, 1 the tanh form of GELU.
+extern "C" int nhv_gemm_fewrows_glu_act_bf16(const void* x, const void* w, void* y, int M, int N, int K, int out_dtype, int act,
+                                             void* stream) {
+  if (sk_check("few-rows gated gemm", x, w, M, N, K, out_dtype)) return 1;
+  NHV_REQUIRE(M <= 16 && (act == 0 || act == 1), "few-rows gated gemm: %d rows (up to 16), activation %d", M, act);
+  NhvGemmFusion f = {};
+  f.glu_act = act;
+  if (nhv_gemm_fewrows_launch(true, x, w, nullptr, y, M, N, K, out_dtype, (hipStream_t)stream, f)) return 1;
+  NHV_LAUNCH_CHECK("gemm_fewrows_glu_act_bf16");
+  return 0;
+}
+
 // ---- products of up to 16 rows that take over the kernels around them (nhv_gemm_fusion.h) ----
 // y = r . (x . w^T) (+ bias), or with glu silu(r . (x . w[0:N]^T)) * (r . (x . w[N:2N]^T)), for 1 <= M <= 16 rows in
 // bfloat16. With ss_in: x is a sum (times its norm's weight) whose rows still lack their scales: r per row from ss_in

@@ -21,4 +21,10 @@ struct NhvGemmFusion {
   const float* ss_in;    // [M, tiles_in]
   int tiles_in;
   float eps;
+  int glu_act;           // what a gated product passes its gate through: 0 SiLU, 1 the tanh form of GELU
 };
+
+__device__ __forceinline__ float nhv_glu_gate(float z, int act) {
+  if (act == 1) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return z / (1.0f + expf(-z));
+}

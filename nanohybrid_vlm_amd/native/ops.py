@@ -681,9 +681,16 @@ class NativeBackend:
         self._call("nhv_scale_rows", _ptr(x), _ptr(squares), squares.shape[1], ctypes.c_float(eps), _ptr(out), x.shape[0],
                    x.shape[1], _stream())
 
-    def gated_linear(self, x, w, out) -> bool:
-        """silu(x Wg^T) * (x Wu^T) in one kernel, if this batch is one for the few-rows kernel; else False."""
+    def gated_linear(self, x, w, out, act: int = 0) -> bool:
+        """act(x Wg^T) * (x Wu^T) in one kernel, if this batch is one for the few-rows kernel; else False.
+        ``act``: 0 SiLU, 1 the tanh form of GELU (up to 16 rows)."""
         M, K = x.shape
+        if act != 0:
+            if x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and M <= self.few_rows:
+                self._call("nhv_gemm_fewrows_glu_act_bf16", _ptr(x), _ptr(w), _ptr(out), M, out.shape[1], K, dtype_code(out),
+                           act, _stream())
+                return True
+            return False
         if (x.dtype == torch.bfloat16 and K % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
                 and (M <= self.few_rows or (M <= 64 and self.own_kernels_only))):
             if M <= self.few_rows and not self.own_kernels_only:
@@ -1080,9 +1087,23 @@ def linear(x, w: torch.Tensor, bias: torch.Tensor | None = None, out_dtype=None,
     return out
 
 
-def gated_linear(x, w: torch.Tensor) -> torch.Tensor:
-    """silu(x . w[:I]^T) * (x . w[I:]^T) for a packed gate | up matrix w[2 I, K]: fused into one kernel for
-    few rows, else the matrix product followed by ``silu_mul``. ``x`` may be a ``Normed`` (see ``linear``)."""
+def gated_linear(x, w: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """act(x . w[:I]^T) * (x . w[I:]^T) for a packed gate | up matrix w[2 I, K]: fused into one kernel for
+    few rows, else the matrix product followed by ``act_mul``. ``x`` may be a ``Normed`` (see ``linear``; with SiLU)."""
+    _need(activation in ACTIVATIONS, lambda: f"gated_linear: activation {activation!r} is not known ({sorted(ACTIVATIONS)} are)")
+    if activation != "silu":
+        x = dense(x)
+        _need(x.dim() == 2 and w.dim() == 2 and w.shape[0] % 2 == 0, "gated_linear: x must be [rows, in] and w [2 * out, in]")
+        _need(x.shape[1] == w.shape[1], lambda: f"gated_linear: x has {x.shape[1]} columns but w has {w.shape[1]}")
+        _dense(x, "gated_linear: x")
+        _dense(w, "gated_linear: w", dtype=x.dtype)
+        dtype_code(x)
+        fused = getattr(backend(), "gated_linear", None)
+        if fused is not None:
+            out = torch.empty((x.shape[0], w.shape[0] // 2), dtype=x.dtype, device=x.device)
+            if fused(x, w, out, ACTIVATIONS[activation]):
+                return out
+        return act_mul(linear(x, w), activation)
     if isinstance(x, Normed):
         normed, x = x, x.summed.weighted
         _need(w.dim() == 2 and w.shape[0] % 2 == 0 and x.shape[1] == w.shape[1], "gated_linear: w must be [2 * out, in]")

@@ -38,7 +38,7 @@ class SwiGLU(Part):
 
     def forward(self, x, step, add_to=None):
         if self.activation != "silu":
-            return ops.linear(ops.act_mul(ops.linear(x, self.gate_up_weight), self.activation), self.down_weight, add_to=add_to)
+            return ops.linear(ops.gated_linear(x, self.gate_up_weight, self.activation), self.down_weight, add_to=add_to)
         return ops.linear(ops.gated_linear(x, self.gate_up_weight), self.down_weight, add_to=add_to)
 
 

@@ -122,6 +122,14 @@ def test_two_layer_norms_of_one_stream_with_pending_additions(where, kernels):
     got = ops.act_mul(gu.to(device), "gelu_tanh")
     want = plain.gelu_tanh(gu[:, :9].double()) * gu[:, 9:].double()
     assert max_abs_diff(got.cpu(), want.float()) <= _tol(dtype, want)
+    # the gate-and-up product with this activation: few rows (one kernel where the rows are bfloat16) and many
+    for rows in (3, 40):
+        x = torch.randn(rows, 24, generator=g).to(_dt(dtype))
+        w = (torch.randn(2 * 16, 24, generator=g) / 24 ** 0.5).to(_dt(dtype))
+        got = ops.gated_linear(x.to(device), w.to(device), "gelu_tanh")
+        both = x.double() @ w.double().T
+        want = plain.gelu_tanh(both[:, :16]) * both[:, 16:]
+        assert max_abs_diff(got.cpu(), want.float()) <= _tol(dtype, want), rows
 
 
 def test_scaled_frequencies_of_the_position_encoding():
