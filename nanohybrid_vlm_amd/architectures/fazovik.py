@@ -68,6 +68,7 @@ class LayerSizes:
     type: str
     mixer: LatentSizes
     mlp: FeedForwardSizes | None
+    spare_norm: bool = False        # a layer without feed-forward whose checkpoint stores a second norm all the same
 
 
 @dataclass(frozen=True)
@@ -158,7 +159,9 @@ def _feed_forward(i: int, mlp) -> FeedForwardSizes | None:
     return f
 
 
-def parse_config(raw: dict) -> FazovikConfig:
+def parse_config(raw: dict, shapes: dict | None = None) -> FazovikConfig:
+    """``shapes``: {stored tensor name: shape} of the checkpoint where there is one: a layer without feed-forward may
+    or may not store its second norm, and only the stored names tell."""
     eps = require(raw.get("norm") or {}, "eps", float)
     if not eps > 0:
         raise ConfigError("config.json: norm.eps must be positive")
@@ -172,7 +175,9 @@ def parse_config(raw: dict) -> FazovikConfig:
             raise ConfigError(f"{_where(i, 'type')}: {kind!r} is not known ('latent_attention' and 'latent_attention_2' are)")
         if not isinstance(m, dict):
             raise ConfigError(f"{_where(i, 'mixer')} is missing")
-        layers.append(LayerSizes(kind, _mixer(i, kind, m, layers), _feed_forward(i, entry.get("mlp"))))
+        mlp = _feed_forward(i, entry.get("mlp"))
+        spare = mlp is None and shapes is not None and f"l{i}.norm2" in shapes
+        layers.append(LayerSizes(kind, _mixer(i, kind, m, layers), mlp, spare))
     pair = None
     bigram = (raw.get("embedding") or {}).get("bigram")
     if bigram is not None:
@@ -210,7 +215,7 @@ def build_spec(cfg: FazovikConfig) -> ModelSpec:
             ff = {"kind": "routed_experts", "hidden_size": cfg.width, "num_experts": f.experts, "top": f.top,
                   "expert_size": f.ff, "activation": "silu"}
         layers.append(LayerSpec(mixer=mixer, feed_forward=ff, norm=norm, position=position,
-                                block={"kind": "parallel_two_norms"}))
+                                block={"kind": "parallel_two_norms", "keeps_unused_norm": layer.spare_norm}))
         order.append(RunEntry(i, cache=a.kv_from))
     embedding = None
     if cfg.pair is not None:
@@ -243,10 +248,11 @@ def checkpoint_names(cfg: FazovikConfig) -> dict[str, WeightSource]:
         for name in ("uq", "uk", "uv", "o"):
             names[ms + name] = WeightSource(md + name + ".weight")
         f = layer.mlp
+        if f is not None or layer.spare_norm:
+            names[src + "norm2"] = WeightSource(dst + "feed_forward_norm.weight")
+            names[src + "norm2.b"] = WeightSource(dst + "feed_forward_norm.bias")
         if f is None:
             continue
-        names[src + "norm2"] = WeightSource(dst + "feed_forward_norm.weight")
-        names[src + "norm2.b"] = WeightSource(dst + "feed_forward_norm.bias")
         fs, fd = src + "mlp.", dst + "feed_forward."
         if f.kind == "dense":
             names[fs + "gate"] = WeightSource(fd + "gate_up.weight", 0, f.ff)
@@ -302,5 +308,6 @@ FAZOVIK = Architecture(
     build_spec=build_spec,
     checkpoint_names=checkpoint_names,
     named_shapes=SHAPES,
+    reads_checkpoint_shapes=True,
 )
 register_architecture(FAZOVIK, replace=True)

@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
 }
 
 extern "C" int nhv_route_topk(const void* logits, void* ids, void* scores, int T, int E, int top, void* stream) {
-  NHV_REQUIRE(T > 0 && E > 0 && top > 0 && top <= E && E <= 8192, "route_topk: bad sizes T=%d E=%d top=%d", T, E, top);
+  NHV_REQUIRE(T > 0 && E > 0 && top > 0 && top <= E && E <= 4096, "route_topk: bad sizes T=%d E=%d (up to 4096) top=%d", T, E, top);
   hipLaunchKernelGGL(route_topk_kernel, dim3((T + 3) / 4), dim3(256), 4 * (size_t)E * sizeof(float), (hipStream_t)stream,
                      (const float*)logits, (int*)ids, (float*)scores, T, E, top);
   NHV_LAUNCH_CHECK("route_topk");

@@ -134,9 +134,12 @@ class ParallelTwoNormsBlock(Part):
     norm_slots = ("mixer_norm", "feed_forward_norm")
     norms_ahead = True            # the model tells the block whether a block follows (``next_norm`` is that block's ``norm``)
 
-    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm):
+    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm, keeps_unused_norm: bool = False):
+        """``keeps_unused_norm``: a block without feed-forward holds its second norm's tensors all the same (a
+        checkpoint that stores them), unused."""
         self.mixer, self.feed_forward = mixer, feed_forward
         self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+        self.keeps_unused_norm = bool(keeps_unused_norm)
         if feed_forward is not None and feed_forward_norm.eps != mixer_norm.eps:
             raise ValueError("the two norms of this block share their statistics and so their eps")
         self.row_dtype = None
@@ -149,8 +152,9 @@ class ParallelTwoNormsBlock(Part):
 
     def children(self):
         out = {"mixer_norm": self.mixer_norm, "mixer": self.mixer}
-        if self.feed_forward is not None:
+        if self.feed_forward is not None or self.keeps_unused_norm:
             out["feed_forward_norm"] = self.feed_forward_norm
+        if self.feed_forward is not None:
             out["feed_forward"] = self.feed_forward
         return out
 

@@ -302,6 +302,21 @@ def test_configuration_and_names(folders):
             arch.parse_config(bad)
 
 
+def test_a_layer_without_feed_forward_may_store_its_second_norm(tmp_path, emulated_kernels):
+    """Such a layer's second norm has nothing to norm for; a checkpoint that stores it all the same is read."""
+    import os
+    from safetensors.torch import save_file
+    folder = str(tmp_path / "m")
+    fc.write_model(folder, fc.CONFIG_F, 3)
+    tensors = fc.random_tensors(fc.CONFIG_F, 3)
+    tensors["l2.norm2"] = torch.ones(fc.CONFIG_F["width"], dtype=torch.bfloat16)
+    tensors["l2.norm2.b"] = torch.zeros(fc.CONFIG_F["width"], dtype=torch.bfloat16)
+    save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(folder, "model.safetensors"))
+    requests = {"a": pc.tokens(fc.CONFIG_F["vocab"], 17, 2)}
+    got = _replay(folder, CPU, pc.in_portions(requests, [5, 1, 11]), page_size=4, max_live=1)
+    _compare(got, _plain_logits(folder, requests), "float32", "portions")
+
+
 # ------------------------------------------------------------------ whole models through the step function
 def _requests(name, lengths):
     vocab = fc.CASES[name][0]["vocab"]
