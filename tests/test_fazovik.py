@@ -317,6 +317,16 @@ def test_a_layer_without_feed_forward_may_store_its_second_norm(tmp_path, emulat
     _compare(got, _plain_logits(folder, requests), "float32", "portions")
 
 
+def test_a_model_without_the_pair_table(tmp_path, emulated_kernels):
+    """Without ``embedding.bigram`` the embedding is the table's rows alone (and no request keeps a previous token)."""
+    config = json.loads(json.dumps(fc.CONFIG_G))
+    del config["embedding"]
+    folder = fc.write_model(str(tmp_path / "m"), config, 5)
+    requests = {"a": pc.tokens(config["vocab"], 14, 3), "b": pc.tokens(config["vocab"], 6, 4)}
+    got = _replay(folder, CPU, pc.interleaved(requests, [3, 1, 4], 2), page_size=4, max_live=2)
+    _compare(got, _plain_logits(folder, requests), "float32", "side by side")
+
+
 # ------------------------------------------------------------------ whole models through the step function
 def _requests(name, lengths):
     vocab = fc.CASES[name][0]["vocab"]
