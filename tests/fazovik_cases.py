@@ -51,9 +51,9 @@ CONFIG_F = _model(131, 44, 1e-5, {"buckets": 37, "mul_cur": 5, "mul_prev": 11}, 
 ])
 # G: stored rows of 64 and 32 entries (the sizes the matrix-core attention kernels take), 17 heads in one layer (more
 # than those kernels' decoding form takes), one expert, one bucket, one head
-CONFIG_G = _model(211, 64, 1e-6, {"buckets": 1, "mul_cur": 3, "mul_prev": 2}, [
+CONFIG_G = _model(211, 64, 2e-6, {"buckets": 1, "mul_cur": 3, "mul_prev": 2}, [
     (_plain(17, 8, 8, 16, 32), _moe(1, 1, 24)),
-    (_rotary(4, 16, 16, 16, 24, 48, 250000.0, {"factor": 2.0, "fast": 32.0, "original": 64, "slow": 1.0}), _dense(96)),
+    (_rotary(4, 16, 16, 16, 24, 48, 40000.0, {"factor": 3.0, "fast": 16.0, "original": 64, "slow": 0.5}), _dense(96)),
     (_plain(1, 16, 24, 8, 32, kv_from=0), _moe(6, 1, 16)),
     (_rotary(6, 8, 32, 8, 16, 32, 1000.0), _moe(4, 4, 8)),
 ])

@@ -134,7 +134,7 @@ def test_two_layer_norms_of_one_stream_with_pending_additions(where, kernels):
 
 def test_scaled_frequencies_of_the_position_encoding():
     from nanohybrid_vlm_amd.parts.positions import YarnFrequencies
-    for rot in ({"dims": 16, "base": 250000.0, "scaling": {"factor": 2.0, "fast": 32.0, "original": 512, "slow": 1.0}},
+    for rot in ({"dims": 12, "base": 30000.0, "scaling": {"factor": 3.0, "fast": 16.0, "original": 256, "slow": 0.5}},
                 {"dims": 8, "base": 100.0, "scaling": {"factor": 8.0, "fast": 4.0, "original": 64, "slow": 2.0}},
                 {"dims": 6, "base": 10000.0}):
         s = rot.get("scaling") or {}
